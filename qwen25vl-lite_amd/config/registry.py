@@ -1,6 +1,6 @@
 """One registry from an architecture's name to its model.
 
-``config.json`` names the architecture (``architectures[0]``, else ``model_type``).  An
+``config.json`` names the architecture (``architectures[0]``, else ``architecture``, else ``model_type``).  An
 architecture is registered as two functions: ``read_config(raw)`` turns the parsed
 ``config.json`` into the architecture's own configuration object (it alone knows its keys), and
 ``build_spec(config)`` turns that into a :class:`~qwen25vl_lite_amd.models.spec.ModelSpec`: the
@@ -86,13 +86,16 @@ def resolve_architecture(name: str) -> Callable:
 
 
 def architecture_name(raw: Dict[str, Any]) -> str:
-    """The registry key a ``config.json`` names: ``architectures[0]``, else ``model_type``."""
+    """The registry key a ``config.json`` names: ``architectures[0]``, else ``architecture``, else
+    ``model_type``."""
     archs = raw.get("architectures") or ()
     if archs:
         return str(archs[0])
+    if raw.get("architecture"):
+        return str(raw["architecture"])
     if raw.get("model_type"):
         return str(raw["model_type"])
-    raise ValueError("config.json names no architecture (neither 'architectures' nor 'model_type')")
+    raise ValueError("config.json names no architecture (none of 'architectures', 'architecture', 'model_type')")
 
 
 def load_config(source) -> Any:

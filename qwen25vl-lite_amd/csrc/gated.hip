@@ -1,0 +1,270 @@
+// Row-wise kernels of gated and normed sublayers: a residual add, a clamped gated activation, a
+// norm over groups of channels with a gate, a per-head output gate, a per-head norm + rotation +
+// cache write for attention whose values may be its unrotated keys, and a soft cap on logits.
+// float32 and bfloat16 storage; all arithmetic is float32.
+#include "common.h"
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// ---------------------------------------------------------------------------------------
+// h[n, :] += delta[n, :]   (float32 sum; delta float32 or bfloat16, or float32 slabs added in order)
+// ---------------------------------------------------------------------------------------
+template <typename TD>
+__global__ void residual_add_kernel(float* __restrict__ h, const TD* __restrict__ delta, long long total, int nslabs,
+                                    long long slab_stride) {
+  const long long step = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step) {
+    float d = ldf<TD>(delta + i);
+    for (int c = 1; c < nslabs; ++c) d += ldf<TD>(delta + (size_t)c * slab_stride + i);
+    h[i] += d;
+  }
+}
+
+extern "C" int qvl_residual_add(void* h, const void* delta, long long total, int delta_dtype, int nslabs,
+                                long long slab_stride, hipStream_t stream) {
+  if (total <= 0) return QVL_OK;
+  if (nslabs < 1 || (nslabs > 1 && delta_dtype != 0)) return QVL_ERR_SHAPE;
+  const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+  if (delta_dtype == 0)
+    hipLaunchKernelGGL(residual_add_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float*)h, (const float*)delta,
+                       total, nslabs, slab_stride);
+  else if (delta_dtype == 1)
+    hipLaunchKernelGGL(residual_add_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (float*)h,
+                       (const bf16_t*)delta, total, nslabs, slab_stride);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Gated activation with clamps: x [N, 2 I] holds the gate branch in columns [0, I) and the linear
+// branch in [I, 2 I);  g = min(gate, limit), u = clamp(lin, -limit, limit) (no clamps if limit <= 0)
+//   out = g * sigmoid(alpha * g) * (u + shift)
+// alpha 1, shift 0, no limit is SwiGLU.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void gated_act_kernel(const T* __restrict__ x, T* __restrict__ out, int I, float alpha, float limit,
+                                 float shift) {
+  const size_t n = blockIdx.y;
+  const T* xr = x + n * 2 * (size_t)I;
+  T* o = out + n * (size_t)I;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < I; i += gridDim.x * blockDim.x) {
+    float g = ldf<T>(xr + i), u = ldf<T>(xr + I + i);
+    if (limit > 0.f) {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+    }
+    stf<T>(o + i, g * sigmoid_f(alpha * g) * (u + shift));
+  }
+}
+
+extern "C" int qvl_gated_act(const void* x, void* out, int N, int I, int dtype, float alpha, float limit, float shift,
+                             hipStream_t stream) {
+  if (N <= 0 || I <= 0) return QVL_OK;
+  if (N > 65535 * 16) return QVL_ERR_LIMIT;
+  // rows go to blockIdx.y (at most 65,535): more rows are launched in pieces
+  const int bx = (I + 255) / 256 > 64 ? 64 : (I + 255) / 256;
+  for (int at = 0; at < N; at += 65535) {
+    const int rows = N - at < 65535 ? N - at : 65535;
+    if (dtype == 0)
+      hipLaunchKernelGGL(gated_act_kernel<float>, dim3(bx, rows), dim3(256), 0, stream,
+                         (const float*)x + (size_t)at * 2 * I, (float*)out + (size_t)at * I, I, alpha, limit, shift);
+    else if (dtype == 1)
+      hipLaunchKernelGGL(gated_act_kernel<bf16_t>, dim3(bx, rows), dim3(256), 0, stream,
+                         (const bf16_t*)x + (size_t)at * 2 * I, (bf16_t*)out + (size_t)at * I, I, alpha, limit, shift);
+    else
+      return QVL_ERR_DTYPE;
+  }
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// logits = cap * tanh(logits / cap), in place, float32
+// ---------------------------------------------------------------------------------------
+__global__ void softcap_kernel(float* __restrict__ x, long long total, float cap) {
+  const long long step = (long long)gridDim.x * blockDim.x;
+  const float inv = 1.0f / cap;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += step)
+    x[i] = cap * tanhf(x[i] * inv);
+}
+
+extern "C" int qvl_softcap(void* x, long long total, float cap, hipStream_t stream) {
+  if (total <= 0) return QVL_OK;
+  if (!(cap > 0.f)) return QVL_ERR_SHAPE;
+  const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+  hipLaunchKernelGGL(softcap_kernel, dim3(blocks), dim3(256), 0, stream, (float*)x, total, cap);
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Norm over groups of `span` consecutive channels, then a gate:
+//   y = x / sqrt(mean_group(x^2) + eps) * w[c % wlen] * act(gate[n, c])
+// x float32 [N, C] (C a multiple of span); gate is read from rows of `gate_stride` values starting at
+// its own pointer; act: 0 no gate, 1 sigmoid, 2 silu.  One block per (group, token).
+// ---------------------------------------------------------------------------------------
+template <typename TG, typename TO>
+__global__ void group_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ w, int wlen,
+                                       const TG* __restrict__ gate, long long gate_stride, TO* __restrict__ out,
+                                       int C, int span, float eps, int act) {
+  __shared__ float red[17];
+  const size_t n = blockIdx.y;
+  const int c0 = blockIdx.x * span;
+  const float* xr = x + n * (size_t)C + c0;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < span; i += blockDim.x) ss += xr[i] * xr[i];
+  const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)span + eps);
+  TO* o = out + n * (size_t)C + c0;
+  const TG* gr = gate ? gate + n * (size_t)gate_stride + c0 : nullptr;
+  for (int i = threadIdx.x; i < span; i += blockDim.x) {
+    float y = (xr[i] * rs) * w[(c0 + i) % wlen];
+    if (act) {
+      const float g = ldf<TG>(gr + i);
+      y *= act == 1 ? sigmoid_f(g) : g * sigmoid_f(g);
+    }
+    stf<TO>(o + i, y);
+  }
+}
+
+extern "C" int qvl_group_norm_gate(const void* x, const void* w, int wlen, const void* gate, long long gate_stride,
+                                   int gate_dtype, void* out, int out_dtype, int N, int C, int span, float eps, int act,
+                                   hipStream_t stream) {
+  if (N <= 0 || C <= 0) return QVL_OK;
+  if (span <= 0 || C % span || wlen <= 0 || (act && !gate) || act < 0 || act > 2) return QVL_ERR_SHAPE;
+  if (C / span > 65535 * 16) return QVL_ERR_LIMIT;
+  const int threads = span >= 1024 ? 1024 : (span + 63) / 64 * 64;
+#define LAUNCH(TG, TO)                                                                                            \
+  for (int at = 0; at < N; at += 65535) {                                                                         \
+    const int rows = N - at < 65535 ? N - at : 65535;                                                             \
+    hipLaunchKernelGGL((group_norm_gate_kernel<TG, TO>), dim3(C / span, rows), dim3(threads), 0, stream,          \
+                       (const float*)x + (size_t)at * C, (const float*)w, wlen,                                   \
+                       gate ? (const TG*)gate + (size_t)at * gate_stride : (const TG*)nullptr, gate_stride,       \
+                       (TO*)out + (size_t)at * C, C, span, eps, act);                                             \
+  }
+  if (gate_dtype == 0 && out_dtype == 0) { LAUNCH(float, float) }
+  else if (gate_dtype == 1 && out_dtype == 1) { LAUNCH(bf16_t, bf16_t) }
+  else if (gate_dtype == 0 && out_dtype == 1) { LAUNCH(float, bf16_t) }
+  else return QVL_ERR_DTYPE;
+#undef LAUNCH
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Per-head output gate: o[n, h, :] *= sigmoid(gate[n, h]);  gate float32 with a row stride.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ o, const float* __restrict__ gate, long long gate_stride, int nh,
+                                 int hd) {
+  const size_t n = blockIdx.x;
+  T* orow = o + n * (size_t)nh * hd;
+  const float* g = gate + n * (size_t)gate_stride;
+  for (int i = threadIdx.x; i < nh * hd; i += blockDim.x) stf<T>(orow + i, ldf<T>(orow + i) * sigmoid_f(g[i / hd]));
+}
+
+extern "C" int qvl_head_gate(void* o, const void* gate, long long gate_stride, int N, int nh, int hd, int dtype,
+                             hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (nh <= 0 || hd <= 0 || gate_stride < nh) return QVL_ERR_SHAPE;
+  if (dtype == 0)
+    hipLaunchKernelGGL(head_gate_kernel<float>, dim3(N), dim3(256), 0, stream, (float*)o, (const float*)gate,
+                       gate_stride, nh, hd);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(head_gate_kernel<bf16_t>, dim3(N), dim3(256), 0, stream, (bf16_t*)o, (const float*)gate,
+                       gate_stride, nh, hd);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Queries and keys of attention with a per-head norm before the rotation:
+//   x [N, stride] float32: nq query heads, then nkv key heads (then nkv value heads unless the
+//   values are the keys as projected: `v_from_k`).
+//   head vector a -> a / sqrt(mean(a^2) + eps) * nw (nw = qw for query heads, kw for key heads; a
+//   null weight skips the norm) -> rotation of the first 2 rot_half channels by the angles whose
+//   cosines and sines are cs[n, f]: pair (2f, 2f+1) if `interleaved`, else (f, f + rot_half).
+//   Queries go to q_out [N, nq hd]; keys into k_cache [pages, nkv, ps, hd] at slots[n]; values
+//   (the key head before norm and rotation, or the value head) into v_cache [pages, nkv, hd, ps].
+// One wave per (token, head); a block holds 4 of them.  hd <= 512.
+// ---------------------------------------------------------------------------------------
+#define QKN_MAX_HD 512
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
+    const float* __restrict__ x, long long x_stride, const float* __restrict__ qw, const float* __restrict__ kw,
+    const float2* __restrict__ cs, const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, int N, int nq, int nkv, int hd, int rot_half, int ps, float eps, int interleaved,
+    int v_from_k, int write_kv) {
+  __shared__ float buf[4][QKN_MAX_HD];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int heads = nq + (write_kv ? (v_from_k ? nkv : 2 * nkv) : 0);
+  const long long item = (long long)blockIdx.x * 4 + wave;
+  if (item >= (long long)N * heads) return;
+  const int n = (int)(item / heads), head = (int)(item % heads);
+  const float* a = x + (size_t)n * x_stride + (size_t)head * hd;
+  float* mine = buf[wave];
+  const int slot = (head >= nq && write_kv) ? slots[n] : -1;
+  const int kind = head < nq ? 0 : (head < nq + nkv ? 1 : 2);   // query, key, value head
+  if (kind != 0 && slot < 0) return;                            // a padding row writes nowhere
+  const size_t page = slot >= 0 ? (size_t)(slot / ps) : 0;
+  const int in_page = slot >= 0 ? slot % ps : 0;
+  if (kind == 2) {
+    const int kvh = head - nq - nkv;
+    T* vrow = v_cache + ((page * nkv + kvh) * hd) * (size_t)ps + in_page;
+    for (int c = lane; c < hd; c += 64) stf<T>(vrow + (size_t)c * ps, a[c]);
+    return;
+  }
+  float ss = 0.f;
+  for (int c = lane; c < hd; c += 64) {
+    const float v = a[c];
+    mine[c] = v;
+    ss += v * v;
+  }
+  const float* nw = kind == 0 ? qw : kw;
+  const float rs = nw ? 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps) : 1.0f;
+  if (kind == 1 && v_from_k) {
+    const int kvh = head - nq;
+    T* vrow = v_cache + ((page * nkv + kvh) * hd) * (size_t)ps + in_page;
+    for (int c = lane; c < hd; c += 64) stf<T>(vrow + (size_t)c * ps, mine[c]);
+  }
+  if (nw)
+    for (int c = lane; c < hd; c += 64) mine[c] = (mine[c] * rs) * nw[c];
+  __builtin_amdgcn_wave_barrier();
+  T* dst = kind == 0 ? q_out + ((size_t)n * nq + head) * hd
+                     : k_cache + ((page * nkv + (head - nq)) * ps + in_page) * (size_t)hd;
+  const float2* csn = cs + (size_t)n * rot_half;
+  for (int c = lane; c < hd; c += 64) {
+    float v = mine[c];
+    if (c < 2 * rot_half) {
+      int f, partner;
+      bool first;
+      if (interleaved) { f = c >> 1; first = !(c & 1); partner = c ^ 1; }
+      else { first = c < rot_half; f = first ? c : c - rot_half; partner = first ? c + rot_half : c - rot_half; }
+      const float2 t = csn[f];
+      const float p = mine[partner];
+      v = first ? v * t.x - p * t.y : v * t.x + p * t.y;
+    }
+    stf<T>(dst + c, v);
+  }
+}
+
+extern "C" int qvl_qk_norm_rope_write(const void* x, long long x_stride, const void* qw, const void* kw, const void* cs,
+                                      const void* slots, void* q_out, void* k_cache, void* v_cache, int N, int nq,
+                                      int nkv, int hd, int rot_half, int ps, float eps, int interleaved, int v_from_k,
+                                      int write_kv, int dtype, hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (nq <= 0 || nkv < 0 || hd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0) return QVL_ERR_SHAPE;
+  if (write_kv && (!slots || !k_cache || !v_cache || nkv <= 0)) return QVL_ERR_SHAPE;
+  if (hd > QKN_MAX_HD) return QVL_ERR_LIMIT;
+  const int heads = nq + (write_kv ? (v_from_k ? nkv : 2 * nkv) : 0);
+  const long long items = (long long)N * heads;
+  const unsigned blocks = (unsigned)((items + 3) / 4);
+#define LAUNCH(T)                                                                                                  \
+  hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(blocks), dim3(256), 0, stream, (const float*)x, x_stride,   \
+                     (const float*)qw, (const float*)kw, (const float2*)cs, (const int*)slots, (T*)q_out,          \
+                     (T*)k_cache, (T*)v_cache, N, nq, nkv, hd, rot_half, ps, eps, interleaved, v_from_k, write_kv)
+  if (dtype == 0) LAUNCH(float);
+  else if (dtype == 1) LAUNCH(bf16_t);
+  else return QVL_ERR_DTYPE;
+#undef LAUNCH
+  return qvl_launch_status();
+}

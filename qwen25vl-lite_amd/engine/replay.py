@@ -35,7 +35,7 @@ ROUND_TO = 64  # a request's token count is rounded up to a multiple of this whe
 
 
 class Replayer:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8):
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 4):
         cfg = load_config(model_dir)
         run_dtype = dtype_from_name(dtype)
         model = build_model(cfg, run_dtype, "cuda:0")
@@ -99,7 +99,8 @@ def main(argv=None) -> int:
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to a multiple of 64)")
     parser.add_argument("--block-size", type=int, default=16)
+    parser.add_argument("--max-live", type=int, default=4, help="requests that may be live at once (state slots)")
     args = parser.parse_args(argv)
-    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size)
+    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size, args.max_live)
     replayer.run(sys.stdin, args.out, sys.stdout)
     return 0

@@ -19,6 +19,12 @@ LIBRARIES = [
     ("gemm_resident", {"RK": 4}),
     ("gemm_split", {}),
     ("peaks", {}),
+    ("gated", {}),
+    # the linear-attention kernels are compiled per key size; any other multiple of 4 up to 256 is
+    # compiled at its first use
+    ("linear_attention", {"LA_DIM": 32}),
+    ("linear_attention", {"LA_DIM": 64}),
+    ("linear_attention", {"LA_DIM": 128}),
     # the matrix-core attention is compiled per head size; these are the sizes the tests and the
     # benchmark use, any other multiple of 16 is compiled at its first use
     ("attention_mfma", {"HD": 128}),

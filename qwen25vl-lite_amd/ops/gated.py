@@ -1,0 +1,139 @@
+"""Python entry points of the row-wise kernels of gated and normed sublayers (``csrc/gated.hip``).
+
+As in :mod:`~qwen25vl_lite_amd.ops.kernels`, every function checks on the host what the kernel and
+its grid assume and launches on the current stream; there is no CPU path.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
+
+__all__ = ["residual_add", "gated_act", "softcap_", "group_norm_gate", "head_gate_", "qk_norm_rope_write"]
+
+_c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+GATE_ACTS = {None: 0, "sigmoid": 1, "silu": 2}
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
+    """``h += delta`` in float32.  ``delta`` is ``[N, H]`` (float32 or bfloat16) or float32
+    ``[slabs, N, H]``, partial sums that are added in slab order."""
+    _dev(h, delta)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [N, H]")
+    nslabs, stride = 1, 0
+    if delta.dim() == 3:
+        _need(delta.dtype == torch.float32 and tuple(delta.shape[1:]) == tuple(h.shape) and delta.is_contiguous(),
+              "slabs of delta must be contiguous float32 [slabs, N, H]")
+        nslabs, stride = delta.shape[0], h.numel()
+    else:
+        _need(delta.shape == h.shape and delta.is_contiguous(), "delta must match h's shape")
+    fn = _fn("gated", "qvl_residual_add", [_c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_ll, _c_ptr])
+    _check(fn(_ptr(h), _ptr(delta), h.numel(), dtype_code(delta.dtype), nslabs, stride, _stream()), "residual_add")
+
+
+def gated_act(x: torch.Tensor, alpha: float = 1.0, limit: Optional[float] = None, shift: float = 0.0) -> torch.Tensor:
+    """``g sigmoid(alpha g) (u + shift)`` for ``x`` of ``[N, 2 I]``, gate branch ``g`` in the first
+    ``I`` columns and linear branch ``u`` in the rest; with ``limit`` the gate is capped from above
+    at it and the linear branch clamped to ``[-limit, limit]`` first."""
+    _dev(x)
+    _need(x.dim() == 2 and x.shape[1] % 2 == 0 and x.is_contiguous(), "x must be contiguous [N, 2 I]")
+    _need(limit is None or limit > 0, "a limit must be positive")
+    n, inter = x.shape[0], x.shape[1] // 2
+    out = torch.empty((n, inter), dtype=x.dtype, device=x.device)
+    fn = _fn("gated", "qvl_gated_act", [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_ptr])
+    _check(fn(_ptr(x), _ptr(out), n, inter, dtype_code(x.dtype), float(alpha), float(limit or 0.0), float(shift),
+              _stream()), "gated_act")
+    return out
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x = cap * tanh(x / cap)`` in place on float32."""
+    _dev(x)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous float32")
+    fn = _fn("gated", "qvl_softcap", [_c_ptr, _c_ll, _c_float, _c_ptr])
+    _check(fn(_ptr(x), x.numel(), float(cap), _stream()), "softcap")
+    return x
+
+
+def group_norm_gate(x: torch.Tensor, weight: torch.Tensor, span: int, eps: float, out_dtype: torch.dtype,
+                    gate: Optional[torch.Tensor] = None, gate_act: Optional[str] = None) -> torch.Tensor:
+    """Every group of ``span`` consecutive channels of float32 ``x [N, C]`` divided by its root
+    mean square, times ``weight[c % len(weight)]``, times ``sigmoid`` or ``silu`` of ``gate[n, c]``
+    (``gate`` may be a view of columns of a wider tensor)."""
+    _dev(x, weight, gate)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [N, C]")
+    n, c = x.shape
+    _need(span > 0 and c % span == 0, "the width must be a multiple of the span")
+    _need(weight.dtype == torch.float32 and weight.dim() == 1 and weight.is_contiguous()
+          and weight.shape[0] in (span, c), "the weight must be float32 of one group's or the row's width")
+    act = GATE_ACTS[gate_act] if gate is not None else 0
+    gstride, gdtype = 0, dtype_code(out_dtype)
+    if gate is not None:
+        _need(gate.shape == (n, c) and gate.stride(1) == 1, "the gate must be [N, C] with contiguous rows")
+        _need(gate.dtype in (torch.float32, out_dtype), "the gate must be float32 or of the output's dtype")
+        gstride, gdtype = gate.stride(0), dtype_code(gate.dtype)
+    out = torch.empty((n, c), dtype=out_dtype, device=x.device)
+    fn = _fn("gated", "qvl_group_norm_gate", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ll, _c_int, _c_ptr, _c_int, _c_int,
+                                               _c_int, _c_int, _c_float, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(weight), weight.shape[0], _ptr(gate), gstride, gdtype, _ptr(out), dtype_code(out_dtype),
+              n, c, int(span), float(eps), act, _stream()), "group_norm_gate")
+    return out
+
+
+def head_gate_(o: torch.Tensor, gate: torch.Tensor, num_heads: int) -> torch.Tensor:
+    """``o[n, h, :] *= sigmoid(gate[n, h])`` in place; ``gate`` float32 ``[N, heads]``, possibly a
+    view of columns of a wider tensor."""
+    _dev(o, gate)
+    n = o.shape[0]
+    _need(o.dim() == 2 and o.is_contiguous() and o.shape[1] % num_heads == 0, "o must be contiguous [N, heads hd]")
+    _need(gate.dtype == torch.float32 and gate.shape == (n, num_heads) and gate.stride(1) == 1,
+          "gate must be float32 [N, heads] with contiguous rows")
+    fn = _fn("gated", "qvl_head_gate", [_c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(o), _ptr(gate), gate.stride(0), n, num_heads, o.shape[1] // num_heads, dtype_code(o.dtype),
+              _stream()), "head_gate")
+    return o
+
+
+def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
+                       cs: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                       v_cache: Optional[torch.Tensor], num_q_heads: int, num_kv_heads: int, head_dim: int,
+                       page_size: int, out_dtype: torch.dtype, *, interleaved: bool, values_are_keys: bool) -> torch.Tensor:
+    """Per head: RMS norm over the head (weights ``q_norm`` / ``k_norm`` of ``[head_dim]``, None: no
+    norm), then rotation by the angles whose ``(cos, sin)`` are ``cs [N, rot/2, 2]``: pairs
+    ``(2f, 2f+1)`` if ``interleaved``, else ``(f, f + rot/2)``.  Rotated queries are returned; rotated
+    keys and the values go into the page slots (``slots`` None: queries only).  ``x`` is float32
+    ``[N, >= (nq + nkv (+ nkv)) hd]``: query heads, key heads, and value heads unless
+    ``values_are_keys``, in which case a key head as projected (before norm and rotation) is its own value."""
+    _dev(x, q_norm, k_norm, cs, slots, k_cache, v_cache)
+    nq, nkv, hd = int(num_q_heads), int(num_kv_heads), int(head_dim)
+    write = slots is not None
+    n = x.shape[0]
+    cols = (nq + (nkv * (1 if values_are_keys else 2) if write else 0)) * hd
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] >= cols and x.stride(1) == 1,
+          "x must be float32 [N, at least the heads' columns]")
+    for w in (q_norm, k_norm):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (hd,) and w.is_contiguous()),
+              "a head norm's weight must be float32 [head_dim]")
+    _need(cs.dtype == torch.float32 and cs.dim() == 3 and cs.is_contiguous() and cs.shape[0] >= n
+          and cs.shape[2] == 2 and 2 * cs.shape[1] <= hd, "cs must be float32 [N, rot/2, 2] with rot <= head_dim")
+    if write:
+        _need(slots.dtype == torch.int32 and slots.shape == (n,) and slots.is_contiguous(), "slots must be int32 [N]")
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == v_cache.dtype == out_dtype,
+              "the cache must have the activation dtype")
+        _need(k_cache.is_contiguous() and k_cache.dim() == 4 and tuple(k_cache.shape[1:]) == (nkv, page_size, hd),
+              "k_cache must be [pages, nkv, page_size, hd]")
+        _need(v_cache.is_contiguous() and tuple(v_cache.shape) == (k_cache.shape[0], nkv, hd, page_size),
+              "v_cache must be [pages, nkv, hd, page_size]")
+    q_out = torch.empty((n, nq * hd), dtype=out_dtype, device=x.device)
+    fn = _fn("gated", "qvl_qk_norm_rope_write",
+             [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+              _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), x.stride(0), _ptr(q_norm), _ptr(k_norm), _ptr(cs), _ptr(slots), _ptr(q_out),
+              _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, n, nq, nkv, hd, cs.shape[1],
+              int(page_size), float(eps), int(interleaved), int(values_are_keys), int(write), dtype_code(out_dtype),
+              _stream()), "qk_norm_rope_write")
+    return q_out

@@ -29,7 +29,16 @@ class PagedAttention(Mixer):
     """params: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim``, ``qkv_bias``,
     ``window`` (None: all keys), ``scale`` (None: ``head_dim ** -0.5``, reference text.py:78),
     ``position`` (a :class:`PartSpec` of category ``position``), ``kv_shared`` (True: the layer
-    has no key/value projections and reads the cache another layer wrote)."""
+    has no key/value projections and reads the cache another layer wrote).
+
+    Optional: ``qk_norm_eps`` (a number: queries and keys are RMS-normed per head before the
+    rotation, with weights ``q_norm`` / ``k_norm`` of ``[head_dim]`` shared by the heads),
+    ``values_are_keys`` (there is no value projection: a key head as projected, before norm and
+    rotation, is its own value), ``head_gate`` (each head's output is multiplied by the sigmoid of
+    one number per head, a projection ``g`` of ``[heads, hidden]`` of the mixer's input), ``names``
+    (local names of the tensors' owners, default ``q_proj`` ... ``o_proj``, ``g_proj``, ``q_norm``,
+    ``k_norm``).  A position encoding may ask for interleaved pairs (``interleaved``).  Any of these
+    takes the projection through float32 and one kernel that norms, rotates and writes the cache."""
 
     graph_safe = True
     takes_lazy_norm = True
@@ -45,10 +54,22 @@ class PagedAttention(Mixer):
         scale = params.get("scale")
         self.scale = float(scale) if scale is not None else self.hd ** -0.5
         self.kv_shared = bool(params.get("kv_shared", False))
+        eps = params.get("qk_norm_eps")
+        self.qk_norm_eps: Optional[float] = None if eps is None else float(eps)
+        self.values_are_keys = bool(params.get("values_are_keys", False))
+        self.head_gate = bool(params.get("head_gate", False))
+        names = dict(params.get("names") or {})
+        self.names = {k: names.get(k, d) for k, d in (("q", "q_proj"), ("k", "k_proj"), ("v", "v_proj"), ("o", "o_proj"),
+                                                      ("g", "g_proj"), ("q_norm", "q_norm"), ("k_norm", "k_norm"))}
+        self.q_norm: Optional[torch.Tensor] = None
+        self.k_norm: Optional[torch.Tensor] = None
         if self.nq % self.nkv:
             raise ValueError(f"{self.nq} heads are not a multiple of {self.nkv} key/value heads")
         pos: PartSpec = params["position"]
         self.position = build_part("position", pos, dtype, device)
+        self.interleaved = bool(getattr(self.position, "interleaved", False))
+        self.normed_path = (self.qk_norm_eps is not None or self.values_are_keys or self.head_gate
+                            or self.interleaved)
         self.w_in: Optional[torch.Tensor] = None
         self.b_in: Optional[torch.Tensor] = None
         self.w_out: Optional[torch.Tensor] = None
@@ -56,38 +77,65 @@ class PagedAttention(Mixer):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(self.nkv, self.hd, self.window)
 
-    def param_specs(self) -> Dict[str, ParamSpec]:
-        specs = {"q_proj.weight": ParamSpec((self.nq * self.hd, self.hidden))}
+    def _projections(self):
+        """``(role, rows)`` of the matrices stacked into the input product, in order."""
+        out = [("q", self.nq * self.hd)]
         if not self.kv_shared:
-            specs["k_proj.weight"] = ParamSpec((self.nkv * self.hd, self.hidden))
-            specs["v_proj.weight"] = ParamSpec((self.nkv * self.hd, self.hidden))
+            out.append(("k", self.nkv * self.hd))
+            if not self.values_are_keys:
+                out.append(("v", self.nkv * self.hd))
+        return out
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        n = self.names
+        specs = {}
+        for role, rows in self._projections():
+            specs[f"{n[role]}.weight"] = ParamSpec((rows, self.hidden))
         if self.qkv_bias:
-            specs["q_proj.bias"] = ParamSpec((self.nq * self.hd,), "vector")
+            for role, rows in self._projections():
+                specs[f"{n[role]}.bias"] = ParamSpec((rows,), "vector")
+        if self.qk_norm_eps is not None:
+            specs[f"{n['q_norm']}.weight"] = ParamSpec((self.hd,), "vector", init="around_one")
             if not self.kv_shared:
-                specs["k_proj.bias"] = ParamSpec((self.nkv * self.hd,), "vector")
-                specs["v_proj.bias"] = ParamSpec((self.nkv * self.hd,), "vector")
-        specs["o_proj.weight"] = ParamSpec((self.hidden, self.nq * self.hd))
+                specs[f"{n['k_norm']}.weight"] = ParamSpec((self.hd,), "vector", init="around_one")
+        if self.head_gate:
+            specs[f"{n['g']}.weight"] = ParamSpec((self.nq, self.hidden))
+        specs[f"{n['o']}.weight"] = ParamSpec((self.hidden, self.nq * self.hd))
         return specs
 
     def load(self, tensors):
-        names = ["q_proj"] if self.kv_shared else ["q_proj", "k_proj", "v_proj"]
-        # One product for q, k and v: the three matrices are stacked by rows.
-        self.w_in = torch.cat([tensors[f"{n}.weight"] for n in names], dim=0).contiguous()
-        self.b_in = torch.cat([tensors[f"{n}.bias"] for n in names]).contiguous() if self.qkv_bias else None
-        self.w_out = tensors["o_proj.weight"]
+        n = self.names
+        roles = [role for role, _ in self._projections()]
+        # One product for q, k and v (and the heads' gate): the matrices are stacked by rows.
+        mats = [tensors[f"{n[r]}.weight"] for r in roles]
+        bias = [tensors[f"{n[r]}.bias"] for r in roles] if self.qkv_bias else None
+        if self.head_gate:
+            mats.append(tensors[f"{n['g']}.weight"])
+            if bias is not None:
+                bias.append(torch.zeros(self.nq, dtype=bias[0].dtype, device=bias[0].device))
+        self.w_in = torch.cat(mats, dim=0).contiguous()
+        self.b_in = torch.cat(bias).contiguous() if bias is not None else None
+        self.w_out = tensors[f"{n['o']}.weight"]
+        if self.qk_norm_eps is not None:
+            self.q_norm = tensors[f"{n['q_norm']}.weight"]
+            self.k_norm = tensors.get(f"{n['k_norm']}.weight")
 
     def named_weights(self) -> Dict[str, torch.Tensor]:
         """Views of the stacked tensors under their checkpoint names."""
+        n = self.names
         out, row = {}, 0
-        for name, heads in (("q_proj", self.nq), ("k_proj", self.nkv), ("v_proj", self.nkv)):
-            if self.kv_shared and name != "q_proj":
-                continue
-            rows = heads * self.hd
-            out[f"{name}.weight"] = self.w_in[row:row + rows]
+        for role, rows in self._projections():
+            out[f"{n[role]}.weight"] = self.w_in[row:row + rows]
             if self.b_in is not None:
-                out[f"{name}.bias"] = self.b_in[row:row + rows]
+                out[f"{n[role]}.bias"] = self.b_in[row:row + rows]
             row += rows
-        out["o_proj.weight"] = self.w_out
+        if self.head_gate:
+            out[f"{n['g']}.weight"] = self.w_in[row:row + self.nq]
+        if self.q_norm is not None:
+            out[f"{n['q_norm']}.weight"] = self.q_norm
+        if self.k_norm is not None:
+            out[f"{n['k_norm']}.weight"] = self.k_norm
+        out[f"{n['o']}.weight"] = self.w_out
         return out
 
     def forward(self, x: torch.Tensor, step: StepContext, slot: LayerSlot) -> torch.Tensor:
@@ -99,10 +147,31 @@ class PagedAttention(Mixer):
             raise RuntimeError("a layer without key/value projections must read another layer's cache, "
                                "and a layer with them must write its own")
         inv_freq, freq_row = self.position.rotary_tables(self.hd)
+        if self.normed_path:
+            return self._forward_normed(x, step, group, slot, write, inv_freq, freq_row)
         q = self._project_few_rows(x, step, group, slot, write, inv_freq, freq_row)
         if q is None:
             q = self._project(x, step, group, slot, write, inv_freq, freq_row)
         o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
+        return linear_into(step.residual, o, self.w_out)
+
+    def _forward_normed(self, x, step, group, slot, write, inv_freq, freq_row):
+        """The path with a per-head norm, interleaved pairs, keys as values or a gate per head: the
+        stacked projection leaves its product in float32, one kernel norms and rotates queries and
+        keys and writes keys and values into the pages, and the gate multiplies the heads' outputs."""
+        from ..ops import gated
+
+        proj = linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
+        cs = self._rotation_table(step, inv_freq, freq_row, proj.shape[0])
+        q = gated.qk_norm_rope_write(
+            proj, self.q_norm, self.k_norm, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0, cs,
+            group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
+            self.nq, self.nkv, self.hd, group.page_size, self.dtype, interleaved=self.interleaved,
+            values_are_keys=self.values_are_keys)
+        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
+        if self.head_gate:
+            at = self.w_in.shape[0] - self.nq
+            gated.head_gate_(o, proj[:, at:at + self.nq], self.nq)
         return linear_into(step.residual, o, self.w_out)
 
     def _project(self, x, step, group, slot, write, inv_freq, freq_row) -> torch.Tensor:

@@ -2,11 +2,11 @@
 
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 from .base import Block, LayerSlot, Part, PartSpec, ResidualStream, StepContext, build_part, register_part
 
-__all__ = ["PreNormBlock"]
+__all__ = ["PreNormBlock", "ParallelBlock"]
 
 
 class PreNormBlock(Block):
@@ -43,4 +43,46 @@ class PreNormBlock(Block):
         return stream
 
 
+class ParallelBlock(Block):
+    """``x = norm(h); h += mixer(x) + ffn(x)``: one norm, both sublayers read its output.
+
+    params: ``norm``, ``mixer`` (:class:`PartSpec` each), ``ffn`` (a :class:`PartSpec`, or None
+    for a layer without a feed-forward) and ``names``, the checkpoint sub-name of each.  The
+    normalised rows are computed before either sublayer runs, so a sublayer's last product may add
+    into ``h`` in place; what a sublayer returns instead is added in float32, the first result by a
+    kernel of its own, the last one by the next norm's kernel.
+    """
+
+    graph_safe = True
+
+    def __init__(self, params, dtype, device):
+        super().__init__(dtype, device)
+        self.norm = build_part("norm", params["norm"], dtype, device)
+        self.mixer = build_part("mixer", params["mixer"], dtype, device)
+        self.ffn: Optional[Part] = None if params.get("ffn") is None else build_part("ffn", params["ffn"], dtype, device)
+        self.names: Dict[str, str] = dict(params["names"])
+
+    def sub_parts(self) -> Dict[str, Part]:
+        parts = {self.names["norm"]: self.norm, self.names["mixer"]: self.mixer}
+        if self.ffn is not None:
+            parts[self.names["ffn"]] = self.ffn
+        return parts
+
+    def forward(self, stream: ResidualStream, step: StepContext, slot: LayerSlot) -> ResidualStream:
+        from ..ops.gated import residual_add
+
+        x = self.norm.forward(stream)        # never lazily: h changes before the second reader would look
+        step.residual = stream.h
+        y = self.mixer.forward(x, step, slot)
+        if self.ffn is None:
+            stream.pending = y
+        else:
+            if y is not None:
+                residual_add(stream.h, y)
+            stream.pending = self.ffn.forward(x, step)
+        step.residual = None
+        return stream
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)

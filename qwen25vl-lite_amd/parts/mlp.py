@@ -9,7 +9,7 @@ import torch
 from ..ops.linear import gate_up_swiglu, linear_into
 from .base import FeedForward, ParamSpec, StepContext, register_part
 
-__all__ = ["SwiGLU"]
+__all__ = ["SwiGLU", "ClampedGatedFF"]
 
 
 class SwiGLU(FeedForward):
@@ -61,4 +61,58 @@ class SwiGLU(FeedForward):
         return linear_into(step.residual if step is not None else None, act, self.w_down)
 
 
+class ClampedGatedFF(FeedForward):
+    """``down(g sigmoid(alpha g) (u + shift))`` with ``g = min(gate(x), limit)`` and
+    ``u = clamp(up(x), -limit, limit)``, no biases.
+
+    params: ``hidden_size``, ``intermediate_size``, ``alpha`` (default 1), ``limit`` (None: no
+    clamps), ``shift`` (default 0), ``names`` (local names of the gate, up and down matrices;
+    default ``gate_proj``, ``up_proj``, ``down_proj``).
+    """
+
+    graph_safe = True
+
+    def __init__(self, params, dtype, device):
+        super().__init__(dtype, device)
+        self.hidden = int(params["hidden_size"])
+        self.inter = int(params["intermediate_size"])
+        self.alpha = float(params.get("alpha", 1.0))
+        limit = params.get("limit")
+        self.limit = None if limit is None else float(limit)
+        if self.limit is not None and not self.limit > 0:
+            raise ValueError("the clamp limit of a feed-forward must be positive")
+        self.shift = float(params.get("shift", 0.0))
+        names = dict(params.get("names") or {})
+        self.names = {k: names.get(k, f"{k}_proj") for k in ("gate", "up", "down")}
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {
+            f"{self.names['gate']}.weight": ParamSpec((self.inter, self.hidden)),
+            f"{self.names['up']}.weight": ParamSpec((self.inter, self.hidden)),
+            f"{self.names['down']}.weight": ParamSpec((self.hidden, self.inter)),
+        }
+
+    def load(self, tensors):
+        # gate and up share their input: one product of [2 I, H], gate rows first
+        self.w_gate_up = torch.cat([tensors[f"{self.names['gate']}.weight"], tensors[f"{self.names['up']}.weight"]],
+                                   dim=0).contiguous()
+        self.w_down = tensors[f"{self.names['down']}.weight"]
+
+    def named_weights(self) -> Dict[str, torch.Tensor]:
+        return {f"{self.names['gate']}.weight": self.w_gate_up[:self.inter],
+                f"{self.names['up']}.weight": self.w_gate_up[self.inter:],
+                f"{self.names['down']}.weight": self.w_down}
+
+    def forward(self, x, step: StepContext):
+        from ..ops.gated import gated_act
+        from ..ops.linear import linear
+
+        both = linear(x, self.w_gate_up)
+        act = gated_act(both if both.is_contiguous() else both.contiguous(), self.alpha, self.limit, self.shift)
+        return linear_into(step.residual if step is not None else None, act, self.w_down)
+
+
 register_part("ffn", "swiglu", SwiGLU)
+register_part("ffn", "clamped_gated", ClampedGatedFF)

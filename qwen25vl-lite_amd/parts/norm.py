@@ -14,10 +14,11 @@ __all__ = ["RMSNorm"]
 
 
 class RMSNorm(Norm):
-    """``x * rsqrt(mean(x^2) + eps) * weight`` with the statistics in float32 and ``eps``
-    inside the root; the weight is used as stored (not ``1 + weight``).
+    """``x * rsqrt(mean(x^2) + eps) * (offset + weight)`` with the statistics in float32 and
+    ``eps`` inside the root.  ``offset`` 0 uses the weight as stored; ``offset`` 1 is a weight
+    stored around zero (the gain is formed once, in float32, when the weight arrives).
 
-    params: ``size`` (row width), ``eps``.
+    params: ``size`` (row width), ``eps``, ``offset`` (default 0).
     """
 
     graph_safe = True
@@ -26,13 +27,15 @@ class RMSNorm(Norm):
         super().__init__(dtype, device)
         self.size = int(params["size"])
         self.eps = float(params["eps"])
-        self.weight: Optional[torch.Tensor] = None
+        self.offset = float(params.get("offset", 0.0))
+        self.weight: Optional[torch.Tensor] = None    # the gain: offset + stored weight
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.size,), "vector", init="around_one")}
+        return {"weight": ParamSpec((self.size,), "vector", init="normal" if self.offset else "around_one")}
 
     def load(self, tensors):
-        self.weight = tensors["weight"]
+        stored = tensors["weight"]
+        self.weight = stored + self.offset if self.offset else stored
 
     def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
         if (lazy and rows is None and stream.pending is None and self.dtype == torch.bfloat16

@@ -13,13 +13,14 @@ of ``inv_freq`` and ``freq_row``:
 
 from __future__ import annotations
 
+import math
 from typing import Tuple
 
 import torch
 
 from .base import PositionEncoding, register_part
 
-__all__ = ["MRoPE", "RoPE1D", "inverse_frequencies"]
+__all__ = ["MRoPE", "RoPE1D", "inverse_frequencies", "rescale_frequencies"]
 
 
 def inverse_frequencies(rotary_dim: int, theta: float) -> torch.Tensor:
@@ -62,8 +63,23 @@ class MRoPE(PositionEncoding):
         return self._tables[head_dim]
 
 
+def rescale_frequencies(freqs: torch.Tensor, factor: float, low: float, high: float, original: int) -> torch.Tensor:
+    """Frequencies stretched for contexts beyond the ``original`` length, by wavelength
+    ``l = 2 pi / f``: ``l < original / high`` keeps ``f``; ``l > original / low`` gives ``f / factor``;
+    between the two, with ``s = (original / l - low) / (high - low)``, the blend
+    ``(1 - s) f / factor + s f``.  Computed in float64."""
+    f = freqs.to(torch.float64)
+    wavelength = 2.0 * math.pi / f
+    s = ((original / wavelength - low) / (high - low)).clamp(0.0, 1.0)
+    blended = (1.0 - s) * f / factor + s * f
+    return torch.where(wavelength < original / high, f, torch.where(wavelength > original / low, f / factor, blended))
+
+
 class RoPE1D(PositionEncoding):
-    """params: ``theta``, optional ``rotary_dim`` (default: the whole head)."""
+    """params: ``theta``, optional ``rotary_dim`` (default: the whole head), optional ``scaling``
+    (``factor``, ``low``, ``high``, ``original``: see :func:`rescale_frequencies`), optional
+    ``interleaved`` (True: channel 2f is rotated with channel 2f+1; default: f with f + rot/2.  The
+    kernel that rotates reads it from the encoding)."""
 
     num_rows = 1
 
@@ -73,18 +89,29 @@ class RoPE1D(PositionEncoding):
         super().__init__(dtype, device)
         self.theta = float(params["theta"])
         self.rotary_dim = params.get("rotary_dim")
+        self.interleaved = bool(params.get("interleaved", False))
+        sc = params.get("scaling")
+        self.scaling = None if not sc else (float(sc["factor"]), float(sc["low"]), float(sc["high"]),
+                                            int(sc["original"]))
+        if self.scaling is not None and not (self.scaling[0] > 0 and self.scaling[2] > self.scaling[1]):
+            raise ValueError("frequency scaling needs a positive factor and high > low")
         self._tables = {}
 
     def table_key(self, head_dim: int):
-        return ("rope", self.theta, self.rotary_dim, head_dim)
+        return ("rope", self.theta, self.rotary_dim, self.scaling, head_dim)
 
     def rotary_tables(self, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
         if head_dim not in self._tables:
             rot = int(self.rotary_dim) if self.rotary_dim is not None else head_dim
             if rot % 2 or rot > head_dim:
                 raise ValueError(f"rotary_dim {rot} must be even and at most the head size {head_dim}")
+            if self.scaling is None:
+                freqs = inverse_frequencies(rot, self.theta)
+            else:
+                idx = torch.arange(0, rot, 2, dtype=torch.float64)
+                freqs = rescale_frequencies(float(self.theta) ** (-idx / rot), *self.scaling).to(torch.float32)
             self._tables[head_dim] = (
-                inverse_frequencies(rot, self.theta).to(self.device),
+                freqs.to(self.device),
                 torch.zeros(rot // 2, dtype=torch.int32, device=self.device),
             )
         return self._tables[head_dim]

@@ -38,9 +38,10 @@ class TokenTable(Embedding):
 
 
 class LinearHead(Head):
-    """``x @ weight.T`` in float32, ``weight`` being ``[vocab, hidden]`` or the tied token table.
+    """``x @ weight.T`` in float32, ``weight`` being ``[vocab, hidden]`` or the tied token table;
+    with ``softcap`` c the logits become ``c tanh(logits / c)``.
 
-    params: ``vocab_size``, ``hidden_size``.
+    params: ``vocab_size``, ``hidden_size``, optional ``softcap``.
     """
 
     graph_safe = True
@@ -48,6 +49,8 @@ class LinearHead(Head):
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
+        cap = params.get("softcap")
+        self.softcap = float(cap) if cap else None
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -62,7 +65,11 @@ class LinearHead(Head):
         self.weight = embedding.table
 
     def forward(self, x, step):
-        return linear(x, self.weight, out_dtype=torch.float32)
+        logits = linear(x, self.weight, out_dtype=torch.float32)
+        if self.softcap is not None:
+            from ..ops.gated import softcap_
+            logits = softcap_(logits if logits.is_contiguous() else logits.contiguous(), self.softcap)
+        return logits
 
 
 register_part("embedding", "token_table", TokenTable)
