@@ -50,6 +50,27 @@ def decoder_config(layers=None, size="7b"):
     return raw
 
 
+def gogudra_config(layers, size="7b", order=("gla", "gla", "lightning", "attention")):
+    """A Gogudra decoder with the width, feed-forward size, head counts and vocabulary of one of SIZES:
+    layers in the given order (repeated), heads of 128 channels (gated linear attention: keys of 64),
+    every layer with its feed-forward."""
+    s = SIZES[size]
+    nh, nkv, hd = s["num_attention_heads"], s["num_key_value_heads"], 128
+    mlp = {"kind": "dense", "ff": s["intermediate_size"], "limit": 7.0}
+    mixers = {
+        "gla": {"heads": nh, "dim": hd // 2, "vdim": hd, "tau": 16.0, "rank": 16},
+        "lightning": {"heads": nh, "dim": hd, "vdim": hd,
+                      "decay": [float(1.0 - 2.0 ** (-5.0 - 3.0 * i / max(1, nh - 1))) for i in range(nh)]},
+        "attention": {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                      "rot": {"base": 500000.0, "dims": hd // 2,
+                              "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+    }
+    return {"architecture": "Gogudra", "width": s["hidden_size"], "vocab": s["vocab_size"], "norm": {"eps": 1e-6},
+            "logit_softcap": 30.0,
+            "layers": [{"type": order[i % len(order)], "mixer": mixers[order[i % len(order)]], "mlp": mlp}
+                       for i in range(int(layers))]}
+
+
 def step_bytes(t, batch, ctx, bytes_per_value=2):
     """Bytes a decode step has to read: every weight it uses once (all layers and the head; of the
     embedding only the rows looked up) and the keys and values of the live requests."""
@@ -204,6 +225,11 @@ def main(argv=None) -> int:
     ap.add_argument("--attention", type=int, nargs="+", metavar="TOKENS",
                     help="instead: the prefill attention alone (one request of that many tokens in one step, the "
                          "chosen size's heads, bfloat16, pages in shuffled order), microseconds and TFLOP/s for each length")
+    ap.add_argument("--design", choices=["gogudra"],
+                    help="instead: prefill (2,048 tokens) and decode throughput of this design at the chosen size's "
+                         "width, heads and feed-forward (random weights), beside the Qwen2.5-VL decoder with as many layers")
+    ap.add_argument("--order", default="gla,gla,lightning,attention",
+                    help="with --design: the mixers of successive layers, repeated")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-lookahead", action="store_true",
                     help="do not queue the next decode step before the running one's tokens are known")
@@ -227,8 +253,11 @@ def main(argv=None) -> int:
     from qwen25vl_lite_amd.config import dtype_from_name
     from qwen25vl_lite_amd.weights import fill_random
 
+    if args.design and not args.layers:
+        args.layers = 8
     cfg = Qwen25VLConfig.from_dict(decoder_config(args.layers, args.size))
     t = cfg.text_config
+    vocab = t.vocab_size
     dtype = dtype_from_name(args.dtype)
     model = build_model(cfg, dtype, "cuda:0")
     fill_random(model, seed=0)
@@ -247,7 +276,7 @@ def main(argv=None) -> int:
         return LLMEngine(runner, ecfg), runner
 
     def prompt(n):
-        return torch.randint(0, t.vocab_size, (n,), generator=gen).tolist()
+        return torch.randint(0, vocab, (n,), generator=gen).tolist()
 
     def decode_rate(batch, steps, warmup):
         budget = max(4096, batch)
@@ -295,6 +324,27 @@ def main(argv=None) -> int:
         torch.cuda.empty_cache()
         return min(times)
 
+    if args.design:
+        from qwen25vl_lite_amd.config import load_config
+        out = {"metric": f"prefill and decode tok/s, {args.design} beside the Qwen2.5-VL decoder "
+                         f"({args.size} sizes, {args.layers} layers, {args.dtype})", "unit": "tokens/s",
+               "order": args.order.split(","), "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
+        steps, warmup = min(args.steps, 64), min(args.warmup, 4)
+        for name in ("qwen25vl", args.design):
+            if name != "qwen25vl":
+                del model
+                torch.cuda.empty_cache()
+                model = build_model(load_config(gogudra_config(args.layers, args.size, tuple(args.order.split(",")))),
+                                    dtype, "cuda:0")
+                fill_random(model, seed=0)
+                torch.cuda.synchronize()
+            sec = prefill_rate(2048)
+            out[name] = {"prefill_tok_s": round(2048 / sec, 1), "prefill_ms": round(sec * 1e3, 3)}
+            if not args.prefill_only:
+                rate, ms, _ = decode_rate(args.batch, steps, warmup)
+                out[name].update({"decode_tok_s": round(rate, 1), "decode_ms_per_step": round(ms, 4)})
+        print(json.dumps(out))
+        return 0
     if args.serving:
         import random
         rng = random.Random(0)

@@ -99,24 +99,33 @@ extern "C" int qvl_softcap(void* x, long long total, float cap, hipStream_t stre
 // ---------------------------------------------------------------------------------------
 // Norm over groups of `span` consecutive channels, then a gate:
 //   y = x / sqrt(mean_group(x^2) + eps) * w[c % wlen] * act(gate[n, c])
-// x float32 [N, C] (C a multiple of span); gate is read from rows of `gate_stride` values starting at
-// its own pointer; act: 0 no gate, 1 sigmoid, 2 silu.  One block per (group, token).
+// x float32 [N, C] (C a multiple of span), or `nslabs` such arrays `slab_stride` apart whose sum, taken
+// in slab order, is x; gate is read from rows of `gate_stride` values starting at its own pointer;
+// act: 0 no gate, 1 sigmoid, 2 silu.  One block per (group, token).
 // ---------------------------------------------------------------------------------------
 template <typename TG, typename TO>
 __global__ void group_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ w, int wlen,
                                        const TG* __restrict__ gate, long long gate_stride, TO* __restrict__ out,
-                                       int C, int span, float eps, int act) {
+                                       int C, int span, float eps, int act, int nslabs, long long slab_stride) {
   __shared__ float red[17];
   const size_t n = blockIdx.y;
   const int c0 = blockIdx.x * span;
   const float* xr = x + n * (size_t)C + c0;
+  auto x_at = [&](int i) {
+    float v = xr[i];
+    for (int s = 1; s < nslabs; ++s) v += xr[(size_t)s * slab_stride + i];
+    return v;
+  };
   float ss = 0.f;
-  for (int i = threadIdx.x; i < span; i += blockDim.x) ss += xr[i] * xr[i];
+  for (int i = threadIdx.x; i < span; i += blockDim.x) {
+    const float v = x_at(i);
+    ss += v * v;
+  }
   const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)span + eps);
   TO* o = out + n * (size_t)C + c0;
   const TG* gr = gate ? gate + n * (size_t)gate_stride + c0 : nullptr;
   for (int i = threadIdx.x; i < span; i += blockDim.x) {
-    float y = (xr[i] * rs) * w[(c0 + i) % wlen];
+    float y = (x_at(i) * rs) * w[(c0 + i) % wlen];
     if (act) {
       const float g = ldf<TG>(gr + i);
       y *= act == 1 ? sigmoid_f(g) : g * sigmoid_f(g);
@@ -127,9 +136,9 @@ __global__ void group_norm_gate_kernel(const float* __restrict__ x, const float*
 
 extern "C" int qvl_group_norm_gate(const void* x, const void* w, int wlen, const void* gate, long long gate_stride,
                                    int gate_dtype, void* out, int out_dtype, int N, int C, int span, float eps, int act,
-                                   hipStream_t stream) {
+                                   int nslabs, long long slab_stride, hipStream_t stream) {
   if (N <= 0 || C <= 0) return QVL_OK;
-  if (span <= 0 || C % span || wlen <= 0 || (act && !gate) || act < 0 || act > 2) return QVL_ERR_SHAPE;
+  if (span <= 0 || C % span || wlen <= 0 || (act && !gate) || act < 0 || act > 2 || nslabs < 1) return QVL_ERR_SHAPE;
   if (C / span > 65535 * 16) return QVL_ERR_LIMIT;
   const int threads = span >= 1024 ? 1024 : (span + 63) / 64 * 64;
 #define LAUNCH(TG, TO)                                                                                            \
@@ -138,7 +147,7 @@ extern "C" int qvl_group_norm_gate(const void* x, const void* w, int wlen, const
     hipLaunchKernelGGL((group_norm_gate_kernel<TG, TO>), dim3(C / span, rows), dim3(threads), 0, stream,          \
                        (const float*)x + (size_t)at * C, (const float*)w, wlen,                                   \
                        gate ? (const TG*)gate + (size_t)at * gate_stride : (const TG*)nullptr, gate_stride,       \
-                       (TO*)out + (size_t)at * C, C, span, eps, act);                                             \
+                       (TO*)out + (size_t)at * C, C, span, eps, act, nslabs, slab_stride);                        \
   }
   if (gate_dtype == 0 && out_dtype == 0) { LAUNCH(float, float) }
   else if (gate_dtype == 1 && out_dtype == 1) { LAUNCH(bf16_t, bf16_t) }

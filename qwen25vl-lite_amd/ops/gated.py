@@ -61,12 +61,15 @@ def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
 
 def group_norm_gate(x: torch.Tensor, weight: torch.Tensor, span: int, eps: float, out_dtype: torch.dtype,
                     gate: Optional[torch.Tensor] = None, gate_act: Optional[str] = None) -> torch.Tensor:
-    """Every group of ``span`` consecutive channels of float32 ``x [N, C]`` divided by its root
+    """Every group of ``span`` consecutive channels of float32 ``x [N, C]`` (or of the sum of the
+    slabs of ``x [slabs, N, C]``, added in order) divided by its root
     mean square, times ``weight[c % len(weight)]``, times ``sigmoid`` or ``silu`` of ``gate[n, c]``
     (``gate`` may be a view of columns of a wider tensor)."""
     _dev(x, weight, gate)
-    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [N, C]")
-    n, c = x.shape
+    _need(x.dtype == torch.float32 and x.dim() in (2, 3) and x.is_contiguous(),
+          "x must be contiguous float32 [N, C] or [slabs, N, C]")
+    nslabs = x.shape[0] if x.dim() == 3 else 1
+    n, c = x.shape[-2:]
     _need(span > 0 and c % span == 0, "the width must be a multiple of the span")
     _need(weight.dtype == torch.float32 and weight.dim() == 1 and weight.is_contiguous()
           and weight.shape[0] in (span, c), "the weight must be float32 of one group's or the row's width")
@@ -78,9 +81,9 @@ def group_norm_gate(x: torch.Tensor, weight: torch.Tensor, span: int, eps: float
         gstride, gdtype = gate.stride(0), dtype_code(gate.dtype)
     out = torch.empty((n, c), dtype=out_dtype, device=x.device)
     fn = _fn("gated", "qvl_group_norm_gate", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ll, _c_int, _c_ptr, _c_int, _c_int,
-                                               _c_int, _c_int, _c_float, _c_int, _c_ptr])
+                                               _c_int, _c_int, _c_float, _c_int, _c_int, _c_ll, _c_ptr])
     _check(fn(_ptr(x), _ptr(weight), weight.shape[0], _ptr(gate), gstride, gdtype, _ptr(out), dtype_code(out_dtype),
-              n, c, int(span), float(eps), act, _stream()), "group_norm_gate")
+              n, c, int(span), float(eps), act, nslabs, n * c, _stream()), "group_norm_gate")
     return out
 
 

@@ -13,16 +13,19 @@ import torch
 
 from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
 
-__all__ = ["decayed_scan", "MAX_KEY_SIZE"]
+__all__ = ["decayed_scan", "scan_groups", "MAX_KEY_SIZE"]
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 MAX_KEY_SIZE = 256
+LONG_RUN = 64
+BLOCKS_PER_CU = 2
+MIN_ROWS = 4
 
 
 def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_heads: int, dim: int, vdim: int,
                  state: torch.Tensor, cu_q: torch.Tensor, req_slots: torch.Tensor, *,
                  head_decay: Optional[torch.Tensor] = None, z: Optional[torch.Tensor] = None, tau: float = 1.0,
-                 silu: bool = False, q_scale: float = 1.0) -> torch.Tensor:
+                 silu: bool = False, q_scale: float = 1.0, groups: int = 1) -> torch.Tensor:
     """Run every request's tokens of the step through the recurrence, from and into ``state``.
 
     ``proj [N, cols]`` (float32 or bfloat16) holds, per token, ``heads * dim`` query columns from
@@ -31,7 +34,9 @@ def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
     The decay is ``head_decay [heads]`` (float32, one constant per head) or, per token and key
     channel, ``sigmoid(z)^(1/tau)`` for float32 ``z [N, heads * dim]``.  ``cu_q [R + 1]`` bounds each
     request's run of tokens, ``req_slots [R]`` names its row of ``state``.  Returns float32
-    ``[N, heads * vdim]``."""
+    ``[groups, N, heads * vdim]``: with ``groups`` above 1 (2, 4 or 8; the key size must be a multiple
+    of four times it) the key channels are cut into that many groups with blocks of their own, and the
+    output is the sum of the slabs (see :func:`scan_groups`)."""
     _dev(proj, state, cu_q, req_slots, head_decay, z)
     h, d, v = int(num_heads), int(dim), int(vdim)
     n = proj.shape[0]
@@ -54,11 +59,28 @@ def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
         _need(z.dtype == torch.float32 and z.shape == (n, h * d) and z.stride(1) == 1, "z must be float32 [N, heads dim]")
         _need(tau > 0, "tau must be positive")
         zstride = z.stride(0)
-    out = torch.empty((n, h * v), dtype=torch.float32, device=proj.device)
+    _need(groups in (1, 2, 4, 8) and d % (4 * groups) == 0, "groups must be 1, 2, 4 or 8 and divide a quarter of the key size")
+    out = torch.empty((groups, n, h * v), dtype=torch.float32, device=proj.device)
     fn = _fn("linear_attention", "qvl_la_scan",
              [_c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr, _c_ptr, _c_ptr,
-              _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr], {"LA_DIM": d})
+              _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr], {"LA_DIM": d})
     _check(fn(_ptr(proj), proj.stride(0), int(q_off), int(k_off), int(v_off), dtype_code(proj.dtype),
               _ptr(head_decay), _ptr(z), zstride, 1.0 / float(tau), _ptr(state), _ptr(cu_q), _ptr(req_slots),
-              _ptr(out), r, h, d, v, int(silu), float(q_scale), _stream()), "decayed_scan")
+              _ptr(out), out.stride(0), int(groups), r, h, d, v, int(silu), float(q_scale), _stream()), "decayed_scan")
     return out
+
+
+def scan_groups(num_reqs: int, max_run: int, num_heads: int, dim: int, vdim: int, device=None) -> int:
+    """Into how many groups of key channels :func:`decayed_scan` is cut for a step.  A block walks its
+    request's tokens one after the other, so the blocks, not the tokens, have to fill the device: runs
+    of ``LONG_RUN`` tokens or more are cut until there are ``BLOCKS_PER_CU`` blocks a compute unit or
+    a wave is down to ``MIN_ROWS`` rows of the state."""
+    if max_run < LONG_RUN:
+        return 1
+    from .attention_mfma import _compute_units
+    blocks = num_reqs * num_heads * ((vdim + 63) // 64)
+    groups = 1
+    while (groups < 8 and blocks * groups < BLOCKS_PER_CU * _compute_units(device)
+           and dim % (8 * groups) == 0 and dim // (8 * groups) >= MIN_ROWS):
+        groups *= 2
+    return groups

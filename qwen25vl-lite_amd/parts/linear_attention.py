@@ -15,7 +15,7 @@ import torch
 
 from ..ops import gated
 from ..ops.linear import linear, linear_into
-from ..ops.linear_attention import decayed_scan
+from ..ops.linear_attention import decayed_scan, scan_groups
 from .base import LayerSlot, Mixer, ParamSpec, StateNeed, StepContext, register_part
 
 __all__ = ["LinearAttention"]
@@ -136,7 +136,8 @@ class LinearAttention(Mixer):
                        out_dtype=torch.float32)
         o = decayed_scan(proj, 0, hk, 2 * hk, self.heads, self.dim, self.vdim, slot.state, step.cu_q, step.req_slots,
                          head_decay=self.head_decay, z=z, tau=self.tau, silu=self.activation == "silu",
-                         q_scale=self.q_scale)
+                         q_scale=self.q_scale,
+                         groups=scan_groups(step.num_reqs, step.max_q_len, self.heads, self.dim, self.vdim, self.device))
         span = hv if self.norm_kind == "all_heads" else self.vdim
         y = gated.group_norm_gate(o, self.w_norm, span, self.eps, self.dtype,
                                   gate=proj[:, 2 * hk + hv:2 * hk + 2 * hv], gate_act=self.gate_act)

@@ -284,3 +284,32 @@ def test_greedy_generation_through_the_entry_point(graph, folders):
              hip_graph=graph) as llm:
         outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True))
     assert [o.output_token_ids for o in outs] == want
+
+
+def test_scan_cut_into_groups_of_key_channels():
+    """Long runs are spread over more blocks by cutting the key channels into groups whose partial
+    outputs are added afterwards: the same outputs and the same final state."""
+    from qwen25vl_lite_amd.ops.linear_attention import decayed_scan, scan_groups
+    assert scan_groups(1, 512, 4, 64, 64, "cuda:0") > 1 and scan_groups(8, 1, 4, 64, 64, "cuda:0") == 1
+    torch.manual_seed(10)
+    n, h, d, v = 150, 2, 32, 72
+    proj = torch.randn(n, 2 * h * d + h * v + 3).cuda()
+    z = (2 + torch.randn(n, h * d)).cuda()
+    cu = torch.tensor([0, 90, 150], dtype=torch.int32).cuda()
+    slots = torch.tensor([2, 0], dtype=torch.int32).cuda()
+    outs, states = [], []
+    for groups in (1, 2, 8):
+        state = torch.zeros(3, h, d, v).cuda()
+        o = decayed_scan(proj, 0, h * d, 2 * h * d, h, d, v, state, cu, slots, z=z, tau=3.0, q_scale=0.5, groups=groups)
+        assert o.shape == (groups, n, h * v)
+        outs.append(o.sum(0).cpu())
+        states.append(state.cpu())
+    q, k, vv = proj[:, :h * d].cpu().double(), proj[:, h * d:2 * h * d].cpu().double(), proj[:, 2 * h * d:2 * h * d + h * v].cpu().double()
+    decay = torch.exp(torch.nn.functional.logsigmoid(z.cpu().double()) / 3.0)
+    for head in range(h):
+        sl, sv = slice(head * d, (head + 1) * d), slice(head * v, (head + 1) * v)
+        want, s_end = plain.decayed_outer_product_scan(0.5 * q[:90, sl], k[:90, sl], vv[:90, sv], decay[:90, sl])
+        for o, st in zip(outs, states):
+            assert torch.allclose(o[:90, sv].double(), want, atol=1e-4 * want.abs().max().item())
+            assert torch.allclose(st[2, head].double(), s_end, atol=1e-4 * s_end.abs().max().item())
+            assert st[1].abs().max() == 0
