@@ -108,6 +108,112 @@ __global__ __launch_bounds__(256) void la_scan_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Long runs, cut into chunks that are scanned side by side.  With P_t = a_c0 * ... * a_t (per key
+// channel, from the chunk's first token c0 to t, t included) and S' the state before the chunk:
+//   o_t = (scan from a zero state)_t + S'^T (q_t * P_t),      S_end = diag(P_last) S' + U
+// where U is the state the scan from zero ends with.  The scan above runs every chunk as if it were a
+// request (from zeroed rows of a scratch tensor); the kernels below form q_t * P_t and P_last, carry
+// the state from chunk to chunk, and put the second term, a plain float32 matrix product per (chunk,
+// head) done by the caller, back into token order.
+// ---------------------------------------------------------------------------------------
+
+// grid (chunks, H), LA_DIM threads: qp [chunks, H, chunk_len, LA_DIM] (rows past the chunk's end stay
+// as they are), last [chunks, H, LA_DIM].
+template <typename TP, bool CHANNEL_DECAY>
+__global__ void la_prefix_kernel(const TP* __restrict__ proj, long long proj_stride, int q_off,
+                                 const float* __restrict__ head_decay, const float* __restrict__ z,
+                                 long long z_stride, float inv_tau, const int* __restrict__ chunk_cu,
+                                 float* __restrict__ qp, float* __restrict__ last, int H, int chunk_len, int act,
+                                 float q_scale) {
+  const int c = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  const int begin = chunk_cu[c], end = chunk_cu[c + 1];
+  const float fixed_log = CHANNEL_DECAY ? 0.f : logf(head_decay[head]);
+  float acc = 0.f;     // log of the running product
+  float* row = qp + ((size_t)c * H + head) * chunk_len * LA_DIM + d;
+  for (int t = begin; t < end; ++t) {
+    if (CHANNEL_DECAY) {
+      const float zz = z[(size_t)t * z_stride + (size_t)head * LA_DIM + d];
+      acc += (fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * inv_tau;
+    } else {
+      acc += fixed_log;
+    }
+    const float q = la_act(ldf<TP>(proj + (size_t)t * proj_stride + q_off + (size_t)head * LA_DIM + d), act) * q_scale;
+    row[(size_t)(t - begin) * LA_DIM] = q * expf(acc);
+  }
+  last[((size_t)c * H + head) * LA_DIM + d] = expf(acc);
+}
+
+// One thread per element of a head's state: for the request's chunks in order, scratch[c] (the chunk's
+// U) is replaced by the state before the chunk, and the request's slot gets the state after its last.
+__global__ void la_carry_kernel(float* __restrict__ scratch, const float* __restrict__ last, float* __restrict__ state,
+                                const int* __restrict__ req_first, const int* __restrict__ req_slots, int H, int vdim) {
+  const int req = blockIdx.y;
+  const long long per_slot = (long long)H * LA_DIM * vdim;
+  const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= per_slot) return;
+  const long long hd = e / vdim;      // head * LA_DIM + d
+  float* mine = state + (size_t)req_slots[req] * per_slot + e;
+  float S = *mine;
+  for (int c = req_first[req]; c < req_first[req + 1]; ++c) {
+    float* u = scratch + (size_t)c * per_slot + e;
+    const float before = S;
+    S = last[(size_t)c * H * LA_DIM + hd] * S + *u;
+    *u = before;
+  }
+  *mine = S;
+}
+
+// corr [chunks, H, chunk_len, vdim] -> out [N, H * vdim]
+__global__ void la_gather_kernel(const float* __restrict__ corr, const int* __restrict__ chunk_cu,
+                                 float* __restrict__ out, int H, int chunk_len, int vdim) {
+  const int c = blockIdx.x, head = blockIdx.y;
+  const int begin = chunk_cu[c], n = chunk_cu[c + 1] - begin;
+  const float* src = corr + ((size_t)c * H + head) * chunk_len * vdim;
+  for (int i = threadIdx.x; i < n * vdim; i += blockDim.x) {
+    const int t = i / vdim, v = i % vdim;
+    out[((size_t)(begin + t) * H + head) * vdim + v] = src[i];
+  }
+}
+
+extern "C" int qvl_la_prefix(const void* proj, long long proj_stride, int q_off, int proj_dtype, const void* head_decay,
+                             const void* z, long long z_stride, float inv_tau, const void* chunk_cu, void* qp,
+                             void* last, int chunks, int H, int dim, int chunk_len, int act, float q_scale,
+                             hipStream_t stream) {
+  if (chunks <= 0) return QVL_OK;
+  if (dim != LA_DIM || H <= 0 || chunk_len <= 0 || (!head_decay && !z)) return QVL_ERR_SHAPE;
+  if (H > 65535 || LA_DIM > 1024) return QVL_ERR_LIMIT;
+#define LAUNCH(TP, CH)                                                                                              \
+  hipLaunchKernelGGL((la_prefix_kernel<TP, CH>), dim3(chunks, H), dim3(LA_DIM), 0, stream, (const TP*)proj,          \
+                     proj_stride, q_off, (const float*)head_decay, (const float*)z, z_stride, inv_tau,               \
+                     (const int*)chunk_cu, (float*)qp, (float*)last, H, chunk_len, act, q_scale)
+  if (proj_dtype == 0) { if (z) LAUNCH(float, true); else LAUNCH(float, false); }
+  else if (proj_dtype == 1) { if (z) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
+  else return QVL_ERR_DTYPE;
+#undef LAUNCH
+  return qvl_launch_status();
+}
+
+extern "C" int qvl_la_carry(void* scratch, const void* last, void* state, const void* req_first, const void* req_slots,
+                            int R, int H, int dim, int vdim, hipStream_t stream) {
+  if (R <= 0) return QVL_OK;
+  if (dim != LA_DIM || H <= 0 || vdim <= 0) return QVL_ERR_SHAPE;
+  if (R > 65535) return QVL_ERR_LIMIT;
+  const long long per_slot = (long long)H * LA_DIM * vdim;
+  hipLaunchKernelGGL(la_carry_kernel, dim3((unsigned)((per_slot + 255) / 256), R), dim3(256), 0, stream, (float*)scratch,
+                     (const float*)last, (float*)state, (const int*)req_first, (const int*)req_slots, H, vdim);
+  return qvl_launch_status();
+}
+
+extern "C" int qvl_la_gather(const void* corr, const void* chunk_cu, void* out, int chunks, int H, int chunk_len,
+                             int vdim, hipStream_t stream) {
+  if (chunks <= 0) return QVL_OK;
+  if (H <= 0 || H > 65535 || chunk_len <= 0 || vdim <= 0) return QVL_ERR_SHAPE;
+  hipLaunchKernelGGL(la_gather_kernel, dim3(chunks, H), dim3(256), 0, stream, (const float*)corr, (const int*)chunk_cu,
+                     (float*)out, H, chunk_len, vdim);
+  return qvl_launch_status();
+}
+
 extern "C" int qvl_la_key_size() { return LA_DIM; }
 
 // proj: rows of `proj_stride` values holding q (H * LA_DIM columns from q_off), k (from k_off) and v

@@ -7,25 +7,31 @@ request in its slot's row of a float32 tensor ``[slots, heads, dim, vdim]``.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
 
 import torch
 
 from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
 
-__all__ = ["decayed_scan", "scan_groups", "MAX_KEY_SIZE"]
+__all__ = ["decayed_scan", "scan_groups", "chunked_scan", "plan_chunks", "ChunkPlan", "MAX_KEY_SIZE", "CHUNK"]
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 MAX_KEY_SIZE = 256
 LONG_RUN = 64
 BLOCKS_PER_CU = 2
 MIN_ROWS = 4
+CHUNK = 64            # tokens of a chunk when long runs are scanned in chunks side by side
+CHUNKED_FROM = 128    # a step whose longest run has this many tokens or more is scanned that way
 
 
 def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_heads: int, dim: int, vdim: int,
                  state: torch.Tensor, cu_q: torch.Tensor, req_slots: torch.Tensor, *,
                  head_decay: Optional[torch.Tensor] = None, z: Optional[torch.Tensor] = None, tau: float = 1.0,
-                 silu: bool = False, q_scale: float = 1.0, groups: int = 1) -> torch.Tensor:
+                 silu: bool = False, q_scale: float = 1.0, groups: int = 1,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Run every request's tokens of the step through the recurrence, from and into ``state``.
 
     ``proj [N, cols]`` (float32 or bfloat16) holds, per token, ``heads * dim`` query columns from
@@ -60,7 +66,10 @@ def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
         _need(tau > 0, "tau must be positive")
         zstride = z.stride(0)
     _need(groups in (1, 2, 4, 8) and d % (4 * groups) == 0, "groups must be 1, 2, 4 or 8 and divide a quarter of the key size")
-    out = torch.empty((groups, n, h * v), dtype=torch.float32, device=proj.device)
+    if out is None:
+        out = torch.empty((groups, n, h * v), dtype=torch.float32, device=proj.device)
+    _need(out.dtype == torch.float32 and out.shape == (groups, n, h * v) and out.is_contiguous() and out.is_cuda,
+          "out must be contiguous float32 [groups, N, heads vdim]")
     fn = _fn("linear_attention", "qvl_la_scan",
              [_c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr, _c_ptr, _c_ptr,
               _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr], {"LA_DIM": d})
@@ -84,3 +93,70 @@ def scan_groups(num_reqs: int, max_run: int, num_heads: int, dim: int, vdim: int
            and dim % (8 * groups) == 0 and dim // (8 * groups) >= MIN_ROWS):
         groups *= 2
     return groups
+
+
+@dataclass
+class ChunkPlan:
+    """A step's runs cut into chunks: ``chunk_cu [chunks + 1]`` (token bounds, chunks follow one another
+    as the runs do), ``chunk_rows [chunks]`` (0, 1, ...: a chunk's row of the scratch state),
+    ``req_first [R + 1]`` (the first chunk of each request), all int32 on the device."""
+
+    chunks: int
+    chunk_len: int
+    chunk_cu: torch.Tensor
+    chunk_rows: torch.Tensor
+    req_first: torch.Tensor
+
+
+def plan_chunks(cu_q_host: Sequence[int], device, chunk_len: int = CHUNK) -> ChunkPlan:
+    bounds, first = [0], [0]
+    for b, e in zip(cu_q_host[:-1], cu_q_host[1:]):
+        at = b
+        while at < e:
+            at = min(at + chunk_len, e)
+            bounds.append(at)
+        first.append(len(bounds) - 1)
+    n = len(bounds) - 1
+    host = np.concatenate([np.asarray(bounds, np.int32), np.arange(n, dtype=np.int32), np.asarray(first, np.int32)])
+    dev = torch.from_numpy(host).to(device)
+    return ChunkPlan(n, chunk_len, dev[:n + 1], dev[n + 1:2 * n + 1], dev[2 * n + 1:])
+
+
+def chunked_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_heads: int, dim: int, vdim: int,
+                 state: torch.Tensor, plan: ChunkPlan, req_slots: torch.Tensor, *,
+                 head_decay: Optional[torch.Tensor] = None, z: Optional[torch.Tensor] = None, tau: float = 1.0,
+                 silu: bool = False, q_scale: float = 1.0) -> torch.Tensor:
+    """:func:`decayed_scan` for steps with long runs: the chunks of ``plan`` are scanned side by side
+    from zero states, the states are carried from chunk to chunk, and what the state before a chunk
+    adds to the chunk's outputs is one float32 matrix product per (chunk, head), ``(q_t P_t) S``
+    with ``P_t`` the product of the decays from the chunk's first token to ``t``.  Returns float32
+    ``[slabs, N, heads * vdim]`` whose sum over the slabs is the output (the last slab holds the
+    second term)."""
+    h, d, v = int(num_heads), int(dim), int(vdim)
+    n = proj.shape[0]
+    nch, clen = plan.chunks, plan.chunk_len
+    scratch = torch.zeros((nch, h, d, v), dtype=torch.float32, device=proj.device)
+    groups = scan_groups(nch, clen, h, d, v, proj.device)
+    out = torch.empty((groups + 1, n, h * v), dtype=torch.float32, device=proj.device)
+    decayed_scan(proj, q_off, k_off, v_off, h, d, v, scratch, plan.chunk_cu, plan.chunk_rows, head_decay=head_decay,
+                 z=z, tau=tau, silu=silu, q_scale=q_scale, groups=groups, out=out[:groups])
+    qp = torch.zeros((nch, h, clen, d), dtype=torch.float32, device=proj.device)
+    last = torch.empty((nch, h, d), dtype=torch.float32, device=proj.device)
+    defines = {"LA_DIM": d}
+    fn = _fn("linear_attention", "qvl_la_prefix",
+             [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+              _c_int, _c_int, _c_int, _c_float, _c_ptr], defines)
+    _check(fn(_ptr(proj), proj.stride(0), int(q_off), dtype_code(proj.dtype), _ptr(head_decay), _ptr(z),
+              z.stride(0) if z is not None else 0, 1.0 / float(tau), _ptr(plan.chunk_cu), _ptr(qp), _ptr(last), nch, h,
+              d, clen, int(silu), float(q_scale), _stream()), "chunk prefix")
+    r = req_slots.shape[0]
+    _need(plan.req_first.shape[0] == r + 1, "the chunk plan belongs to another step")
+    fn = _fn("linear_attention", "qvl_la_carry", [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                                                   _c_ptr], defines)
+    _check(fn(_ptr(scratch), _ptr(last), _ptr(state), _ptr(plan.req_first), _ptr(req_slots), r, h, d, v, _stream()),
+           "chunk carry")
+    corr = torch.matmul(qp, scratch)          # [chunks, heads, chunk_len, vdim], true float32
+    fn = _fn("linear_attention", "qvl_la_gather", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+             defines)
+    _check(fn(_ptr(corr), _ptr(plan.chunk_cu), _ptr(out[groups]), nch, h, clen, v, _stream()), "chunk gather")
+    return out

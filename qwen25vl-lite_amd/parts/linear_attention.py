@@ -15,7 +15,7 @@ import torch
 
 from ..ops import gated
 from ..ops.linear import linear, linear_into
-from ..ops.linear_attention import decayed_scan, scan_groups
+from ..ops.linear_attention import CHUNKED_FROM, chunked_scan, decayed_scan, plan_chunks, scan_groups
 from .base import LayerSlot, Mixer, ParamSpec, StateNeed, StepContext, register_part
 
 __all__ = ["LinearAttention"]
@@ -134,10 +134,17 @@ class LinearAttention(Mixer):
             low = proj[:, at:at + self.rank]         # a few columns: copied to rows of their own
             z = linear(low.contiguous(), self.w_a2, self.b_a2,
                        out_dtype=torch.float32)
-        o = decayed_scan(proj, 0, hk, 2 * hk, self.heads, self.dim, self.vdim, slot.state, step.cu_q, step.req_slots,
-                         head_decay=self.head_decay, z=z, tau=self.tau, silu=self.activation == "silu",
-                         q_scale=self.q_scale,
-                         groups=scan_groups(step.num_reqs, step.max_q_len, self.heads, self.dim, self.vdim, self.device))
+        how = dict(head_decay=self.head_decay, z=z, tau=self.tau, silu=self.activation == "silu", q_scale=self.q_scale)
+        if step.max_q_len >= CHUNKED_FROM and len(step.cu_q_host) == step.num_reqs + 1:
+            # long runs (never a captured decode step): in chunks side by side; the plan is the step's, shared by layers
+            plan = step.derived.get("la_chunks")
+            if plan is None:
+                plan = step.derived["la_chunks"] = plan_chunks(step.cu_q_host, self.device)
+            o = chunked_scan(proj, 0, hk, 2 * hk, self.heads, self.dim, self.vdim, slot.state, plan, step.req_slots, **how)
+        else:
+            o = decayed_scan(proj, 0, hk, 2 * hk, self.heads, self.dim, self.vdim, slot.state, step.cu_q,
+                             step.req_slots, groups=scan_groups(step.num_reqs, step.max_q_len, self.heads, self.dim,
+                                                                self.vdim, self.device), **how)
         span = hv if self.norm_kind == "all_heads" else self.vdim
         y = gated.group_norm_gate(o, self.w_norm, span, self.eps, self.dtype,
                                   gate=proj[:, 2 * hk + hv:2 * hk + 2 * hv], gate_act=self.gate_act)

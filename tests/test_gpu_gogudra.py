@@ -313,3 +313,32 @@ def test_scan_cut_into_groups_of_key_channels():
             assert torch.allclose(o[:90, sv].double(), want, atol=1e-4 * want.abs().max().item())
             assert torch.allclose(st[2, head].double(), s_end, atol=1e-4 * s_end.abs().max().item())
             assert st[1].abs().max() == 0
+
+
+@pytest.mark.parametrize("channel", [False, True])
+def test_long_runs_scanned_in_chunks(channel):
+    """Runs cut into chunks that are scanned side by side and stitched through the carried state: the
+    same outputs and final states as one scan, for runs that end inside a chunk, a run of one token,
+    and states that do not start at zero."""
+    from qwen25vl_lite_amd.ops.linear_attention import chunked_scan, decayed_scan, plan_chunks
+    torch.manual_seed(11)
+    runs = [150, 1, 64, 70]
+    n, h, d, v = sum(runs), 3, 16, 40
+    proj = torch.randn(n, 2 * h * d + h * v).cuda()
+    z = (1 + 2 * torch.randn(n, h * d)).cuda() if channel else None
+    decay = None if channel else torch.tensor([0.5, 0.97, 1.0]).cuda()
+    bounds = [0]
+    for r in runs:
+        bounds.append(bounds[-1] + r)
+    cu = torch.tensor(bounds, dtype=torch.int32).cuda()
+    slots = torch.tensor([3, 0, 1, 2], dtype=torch.int32).cuda()
+    start = 0.3 * torch.randn(5, h, d, v).cuda()
+    how = dict(head_decay=decay, z=z, tau=2.0, silu=not channel, q_scale=0.7)
+    s1 = start.clone()
+    want = decayed_scan(proj, 0, h * d, 2 * h * d, h, d, v, s1, cu, slots, **how).sum(0)
+    s2 = start.clone()
+    plan = plan_chunks(bounds, "cuda:0", 64)
+    assert plan.chunks == 3 + 1 + 1 + 2 and plan.req_first.tolist() == [0, 3, 4, 5, 7]
+    got = chunked_scan(proj, 0, h * d, 2 * h * d, h, d, v, s2, plan, slots, **how).sum(0)
+    assert torch.allclose(got, want, atol=2e-5 * want.abs().max().item()), (got - want).abs().max()
+    assert torch.allclose(s2, s1, atol=2e-5 * s1.abs().max().item()) and torch.equal(s2[4], start[4])
