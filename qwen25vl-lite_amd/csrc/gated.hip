@@ -6,6 +6,23 @@
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// four consecutive values as float32
+template <typename T> __device__ __forceinline__ float4 ldv4(const T* p);
+template <> __device__ __forceinline__ float4 ldv4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 ldv4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                __uint_as_float(v.y & 0xffff0000u)};
+}
+template <typename T> __device__ __forceinline__ void stv4(T* p, float4 v);
+template <> __device__ __forceinline__ void stv4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void stv4<bf16_t>(bf16_t* p, float4 v) {
+  uint2 o;
+  o.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+  o.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = o;
+}
+
 // ---------------------------------------------------------------------------------------
 // h[n, :] += delta[n, :]   (float32 sum; delta float32 or bfloat16, or float32 slabs added in order)
 // ---------------------------------------------------------------------------------------
@@ -58,9 +75,45 @@ __global__ void gated_act_kernel(const T* __restrict__ x, T* __restrict__ out, i
   }
 }
 
+// The same, four values a thread (I a multiple of 4): one grid-stride loop over all rows.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_act_vec_kernel(const T* __restrict__ x, T* __restrict__ out, int I,
+                                                            long long vectors, float alpha, float limit, float shift) {
+  const int per_row = I >> 2;
+  const long long step = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < vectors; i += step) {
+    const long long n = i / per_row;
+    const int c = (int)(i % per_row) << 2;
+    const T* xr = x + n * 2 * (size_t)I + c;
+    float4 g = ldv4<T>(xr), u = ldv4<T>(xr + I), y;
+    float* gp = &g.x; float* up = &u.x; float* yp = &y.x;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float gg = gp[k], uu = up[k];
+      if (limit > 0.f) {
+        gg = fminf(gg, limit);
+        uu = fminf(fmaxf(uu, -limit), limit);
+      }
+      yp[k] = gg * sigmoid_f(alpha * gg) * (uu + shift);
+    }
+    stv4<T>(out + n * (size_t)I + c, y);
+  }
+}
+
 extern "C" int qvl_gated_act(const void* x, void* out, int N, int I, int dtype, float alpha, float limit, float shift,
                              hipStream_t stream) {
   if (N <= 0 || I <= 0) return QVL_OK;
+  if (I % 4 == 0 && (dtype == 0 || dtype == 1)) {
+    const long long vectors = (long long)N * (I >> 2);
+    const int blocks = (int)((vectors + 255) / 256 > 16384 ? 16384 : (vectors + 255) / 256);
+    if (dtype == 0)
+      hipLaunchKernelGGL(gated_act_vec_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, (float*)out,
+                         I, vectors, alpha, limit, shift);
+    else
+      hipLaunchKernelGGL(gated_act_vec_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)x,
+                         (bf16_t*)out, I, vectors, alpha, limit, shift);
+    return qvl_launch_status();
+  }
   if (N > 65535 * 16) return QVL_ERR_LIMIT;
   // rows go to blockIdx.y (at most 65,535): more rows are launched in pieces
   const int bx = (I + 255) / 256 > 64 ? 64 : (I + 255) / 256;
@@ -134,12 +187,91 @@ __global__ void group_norm_gate_kernel(const float* __restrict__ x, const float*
   }
 }
 
+// The same with a team of TEAM threads (a wave, or the block) per group, four values at a time, the
+// group's values held in registers between the two passes: span a multiple of 4 and at most
+// TEAM * 4 * GN_VEC.  Blocks of 256 threads; blockIdx.x counts teams over all (token, group) pairs.
+#define GN_VEC 4
+
+template <typename TG, typename TO, int TEAM>
+__global__ __launch_bounds__(256) void group_norm_gate_vec_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, int wlen, const TG* __restrict__ gate,
+    long long gate_stride, TO* __restrict__ out, int C, int span, float eps, int act, int nslabs,
+    long long slab_stride, long long items) {
+  __shared__ float red[17];
+  const int team = threadIdx.x / TEAM, lane = threadIdx.x % TEAM;
+  const long long item = (long long)blockIdx.x * (256 / TEAM) + team;
+  const bool live = item < items;               // a whole team at once
+  const int groups = C / span;
+  const size_t n = live ? (size_t)(item / groups) : 0;
+  const int c0 = live ? (int)(item % groups) * span : 0;
+  const float* xr = x + n * (size_t)C + c0;
+  const int nvec = span >> 2;
+  float4 v[GN_VEC];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < GN_VEC; ++j) {
+    const int i = lane + TEAM * j;
+    v[j] = float4{0.f, 0.f, 0.f, 0.f};
+    if (live && i < nvec) {
+      v[j] = ldv4<float>(xr + 4 * i);
+      for (int s = 1; s < nslabs; ++s) {
+        const float4 a = ldv4<float>(xr + (size_t)s * slab_stride + 4 * i);
+        v[j].x += a.x; v[j].y += a.y; v[j].z += a.z; v[j].w += a.w;
+      }
+      ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    }
+  }
+  const float total = TEAM == 64 ? wave_sum(ss) : block_sum(ss, red);
+  if (!live) return;
+  const float rs = 1.0f / sqrtf(total / (float)span + eps);
+  TO* o = out + n * (size_t)C + c0;
+  const TG* gr = gate ? gate + n * (size_t)gate_stride + c0 : nullptr;
+#pragma unroll
+  for (int j = 0; j < GN_VEC; ++j) {
+    const int i = lane + TEAM * j;
+    if (i < nvec) {
+      const int wc = (c0 + 4 * i) % wlen;       // wlen is a multiple of 4 here, so the four stay in one period
+      const float4 ww = ldv4<float>(w + wc);
+      float4 y{(v[j].x * rs) * ww.x, (v[j].y * rs) * ww.y, (v[j].z * rs) * ww.z, (v[j].w * rs) * ww.w};
+      if (act) {
+        const float4 g = ldv4<TG>(gr + 4 * i);
+        if (act == 1) { y.x *= sigmoid_f(g.x); y.y *= sigmoid_f(g.y); y.z *= sigmoid_f(g.z); y.w *= sigmoid_f(g.w); }
+        else { y.x *= g.x * sigmoid_f(g.x); y.y *= g.y * sigmoid_f(g.y); y.z *= g.z * sigmoid_f(g.z); y.w *= g.w * sigmoid_f(g.w); }
+      }
+      stv4<TO>(o + 4 * i, y);
+    }
+  }
+}
+
 extern "C" int qvl_group_norm_gate(const void* x, const void* w, int wlen, const void* gate, long long gate_stride,
                                    int gate_dtype, void* out, int out_dtype, int N, int C, int span, float eps, int act,
                                    int nslabs, long long slab_stride, hipStream_t stream) {
   if (N <= 0 || C <= 0) return QVL_OK;
   if (span <= 0 || C % span || wlen <= 0 || (act && !gate) || act < 0 || act > 2 || nslabs < 1) return QVL_ERR_SHAPE;
   if (C / span > 65535 * 16) return QVL_ERR_LIMIT;
+  // the vector kernel: widths, strides and addresses in steps of four values (16 bytes of float32)
+  const int gbytes = gate_dtype == 0 ? 4 : 2;
+  const bool vec = span % 4 == 0 && wlen % 4 == 0 && span <= 256 * 4 * GN_VEC && slab_stride % 4 == 0 &&
+                   (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+                   (!gate || (gate_stride % 4 == 0 && (uintptr_t)gate % (4 * gbytes) == 0));
+  if (vec) {
+    const long long items = (long long)N * (C / span);
+    const bool wave = span <= 64 * 4 * GN_VEC;
+    const long long blocks = wave ? (items + 3) / 4 : items;
+    if (blocks > 0x7fffffffLL) return QVL_ERR_LIMIT;
+#define LAUNCHV(TG, TO, TEAM)                                                                                      \
+    hipLaunchKernelGGL((group_norm_gate_vec_kernel<TG, TO, TEAM>), dim3((unsigned)blocks), dim3(256), 0, stream,   \
+                       (const float*)x, (const float*)w, wlen, (const TG*)gate, gate_stride, (TO*)out, C, span,    \
+                       eps, act, nslabs, slab_stride, items)
+#define BY_TEAM(TG, TO) if (wave) LAUNCHV(TG, TO, 64); else LAUNCHV(TG, TO, 256)
+    if (gate_dtype == 0 && out_dtype == 0) { BY_TEAM(float, float); }
+    else if (gate_dtype == 1 && out_dtype == 1) { BY_TEAM(bf16_t, bf16_t); }
+    else if (gate_dtype == 0 && out_dtype == 1) { BY_TEAM(float, bf16_t); }
+    else return QVL_ERR_DTYPE;
+#undef BY_TEAM
+#undef LAUNCHV
+    return qvl_launch_status();
+  }
   const int threads = span >= 1024 ? 1024 : (span + 63) / 64 * 64;
 #define LAUNCH(TG, TO)                                                                                            \
   for (int at = 0; at < N; at += 65535) {                                                                         \

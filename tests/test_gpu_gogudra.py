@@ -342,3 +342,39 @@ def test_long_runs_scanned_in_chunks(channel):
     got = chunked_scan(proj, 0, h * d, 2 * h * d, h, d, v, s2, plan, slots, **how).sum(0)
     assert torch.allclose(got, want, atol=2e-5 * want.abs().max().item()), (got - want).abs().max()
     assert torch.allclose(s2, s1, atol=2e-5 * s1.abs().max().item()) and torch.equal(s2[4], start[4])
+
+
+@pytest.mark.parametrize("span, groups", [(7, 3), (24, 5), (128, 2), (1024, 1), (1500, 2), (4100, 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_group_norm_with_gate_at_any_width(span, groups, dtype):
+    """Narrow groups (a wave each), wide ones (a block each), widths that are not a multiple of four,
+    partial sums in slabs, a gate that is a view of a wider tensor."""
+    from qwen25vl_lite_amd.ops.gated import group_norm_gate
+    torch.manual_seed(span)
+    n, c = 5, span * groups
+    slabs = torch.randn(3, n, c)
+    wide = torch.randn(n, c + 8).to(dtype)
+    for weight in (torch.randn(span), torch.randn(c)):
+        for act, fn in (("sigmoid", torch.sigmoid), ("silu", torch.nn.functional.silu)):
+            x = slabs.sum(0).double().view(n, groups, span)
+            want = (plain.unit_rms(x, 1e-3).view(n, c) * weight.double().repeat(c // weight.shape[0])
+                    * fn(wide[:, 8:].double()))
+            got = group_norm_gate(slabs.cuda(), weight.cuda(), span, 1e-3, dtype, gate=wide.cuda()[:, 8:], gate_act=act)
+            tol = 1e-5 if dtype == torch.float32 else 1e-2
+            assert torch.allclose(got.double().cpu(), want, atol=tol * want.abs().max().item(), rtol=tol)
+
+
+@pytest.mark.parametrize("inter", [5, 72, 1000])
+def test_gated_activation_at_any_width(inter):
+    from qwen25vl_lite_amd.ops.gated import gated_act
+    torch.manual_seed(inter)
+    x = 2 * torch.randn(7, 2 * inter)
+    for dtype in (torch.float32, torch.bfloat16):
+        xd = x.to(dtype)
+        g, u = xd[:, :inter].double().clamp(max=0.9), xd[:, inter:].double().clamp(-0.9, 0.9)
+        want = g * torch.sigmoid(1.3 * g) * (u + 0.5)
+        got = gated_act(xd.cuda(), 1.3, 0.9, 0.5).double().cpu()
+        assert torch.allclose(got, want, atol=1e-5 if dtype == torch.float32 else 2e-2)
+        free = gated_act(xd.cuda()).double().cpu()
+        assert torch.allclose(free, torch.nn.functional.silu(xd[:, :inter].double()) * xd[:, inter:].double(),
+                              atol=1e-5 if dtype == torch.float32 else 1e-2, rtol=1e-5 if dtype == torch.float32 else 1e-2)
