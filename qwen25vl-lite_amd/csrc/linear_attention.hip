@@ -118,30 +118,43 @@ __global__ __launch_bounds__(256) void la_scan_kernel(
 // head) done by the caller, back into token order.
 // ---------------------------------------------------------------------------------------
 
-// grid (chunks, H), LA_DIM threads: qp [chunks, H, chunk_len, LA_DIM] (rows past the chunk's end stay
-// as they are), last [chunks, H, LA_DIM].
+// grid (chunks, H), LA_DIM * LA_PARTS threads: qp [chunks, H, chunk_len, LA_DIM] (rows past the chunk's end
+// stay as they are), last [chunks, H, LA_DIM].  The chunk's tokens are cut into LA_PARTS ranges; a thread
+// sums the logarithms of its channel's decays over its range, learns through LDS what the ranges before
+// it add up to, and walks its range again to write q_t * P_t.
+#define LA_PARTS (LA_DIM <= 64 ? 8 : (LA_DIM <= 128 ? 4 : 2))
+
 template <typename TP, bool CHANNEL_DECAY>
 __global__ void la_prefix_kernel(const TP* __restrict__ proj, long long proj_stride, int q_off,
                                  const float* __restrict__ head_decay, const float* __restrict__ z,
                                  long long z_stride, float inv_tau, const int* __restrict__ chunk_cu,
                                  float* __restrict__ qp, float* __restrict__ last, int H, int chunk_len, int act,
                                  float q_scale) {
-  const int c = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  __shared__ float part_sum[LA_PARTS][LA_DIM];
+  const int c = blockIdx.x, head = blockIdx.y, d = threadIdx.x % LA_DIM, part = threadIdx.x / LA_DIM;
   const int begin = chunk_cu[c], end = chunk_cu[c + 1];
+  const int per = (end - begin + LA_PARTS - 1) / LA_PARTS;
+  const int lo = begin + part * per < end ? begin + part * per : end;
+  const int hi = lo + per < end ? lo + per : end;
   const float fixed_log = CHANNEL_DECAY ? 0.f : logf(head_decay[head]);
-  float acc = 0.f;     // log of the running product
+  auto log_decay = [&](int t) {
+    if (!CHANNEL_DECAY) return fixed_log;
+    const float zz = z[(size_t)t * z_stride + (size_t)head * LA_DIM + d];
+    return (fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * inv_tau;
+  };
+  float mine = 0.f;
+  for (int t = lo; t < hi; ++t) mine += log_decay(t);
+  part_sum[part][d] = mine;
+  __syncthreads();
+  float acc = 0.f;     // log of the running product, from the chunk's first token on
+  for (int p = 0; p < part; ++p) acc += part_sum[p][d];
   float* row = qp + ((size_t)c * H + head) * chunk_len * LA_DIM + d;
-  for (int t = begin; t < end; ++t) {
-    if (CHANNEL_DECAY) {
-      const float zz = z[(size_t)t * z_stride + (size_t)head * LA_DIM + d];
-      acc += (fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * inv_tau;
-    } else {
-      acc += fixed_log;
-    }
+  for (int t = lo; t < hi; ++t) {
+    acc += log_decay(t);
     const float q = la_act(ldf<TP>(proj + (size_t)t * proj_stride + q_off + (size_t)head * LA_DIM + d), act) * q_scale;
     row[(size_t)(t - begin) * LA_DIM] = q * expf(acc);
   }
-  last[((size_t)c * H + head) * LA_DIM + d] = expf(acc);
+  if (part == LA_PARTS - 1) last[((size_t)c * H + head) * LA_DIM + d] = expf(acc);
 }
 
 // One thread per element of a head's state: for the request's chunks in order, scratch[c] (the chunk's
@@ -182,9 +195,9 @@ extern "C" int qvl_la_prefix(const void* proj, long long proj_stride, int q_off,
                              hipStream_t stream) {
   if (chunks <= 0) return QVL_OK;
   if (dim != LA_DIM || H <= 0 || chunk_len <= 0 || (!head_decay && !z)) return QVL_ERR_SHAPE;
-  if (H > 65535 || LA_DIM > 1024) return QVL_ERR_LIMIT;
+  if (H > 65535 || LA_DIM * LA_PARTS > 1024) return QVL_ERR_LIMIT;
 #define LAUNCH(TP, CH)                                                                                              \
-  hipLaunchKernelGGL((la_prefix_kernel<TP, CH>), dim3(chunks, H), dim3(LA_DIM), 0, stream, (const TP*)proj,          \
+  hipLaunchKernelGGL((la_prefix_kernel<TP, CH>), dim3(chunks, H), dim3(LA_DIM * LA_PARTS), 0, stream, (const TP*)proj, \
                      proj_stride, q_off, (const float*)head_decay, (const float*)z, z_stride, inv_tau,               \
                      (const int*)chunk_cu, (float*)qp, (float*)last, H, chunk_len, act, q_scale)
   if (proj_dtype == 0) { if (z) LAUNCH(float, true); else LAUNCH(float, false); }
