@@ -7,7 +7,8 @@
 //
 // The scan: a block of four waves owns 64 value channels of one head of one request and walks the
 // request's tokens of this step in order, starting from the state its slot holds and leaving the
-// new state there.  Lane = value channel; each wave keeps LA_DIM / 4 rows of S in registers.
+// new state there.  Lane = value channel; each wave keeps LA_DIM / 4 rows of S in registers (a key
+// size that four does not divide is shared by two waves, or kept by one).
 // Tokens are staged LA_TB at a time: q, k and the decays go to LDS (every lane reads the same
 // word), the four partial sums of o meet in LDS.  The order of every sum is fixed by the sizes
 // alone, so a token's result does not depend on how its sequence was cut into steps or on what
@@ -22,10 +23,11 @@
 #ifndef LA_DIM
 #define LA_DIM 64
 #endif
-#define LA_WAVES 4
+// waves of a block: four share the rows of S where the key size divides by four, else two or one
+#define LA_WAVES (LA_DIM % 4 == 0 ? 4 : (LA_DIM % 2 == 0 ? 2 : 1))
+#define LA_THREADS (64 * LA_WAVES)
 #define LA_TB (LA_DIM > 128 ? 8 : 16)
 
-static_assert(LA_DIM % LA_WAVES == 0, "the key size must be a multiple of 4");
 
 __device__ __forceinline__ float la_act(float z, int act) { return act ? z / (1.0f + expf(-z)) : z; }
 
@@ -35,7 +37,7 @@ __device__ __forceinline__ float la_decay(float z, float inv_tau) {
 }
 
 template <typename TP, bool CHANNEL_DECAY, int G>
-__global__ __launch_bounds__(256) void la_scan_kernel(
+__global__ __launch_bounds__(LA_THREADS) void la_scan_kernel(
     const TP* __restrict__ proj, long long proj_stride, int q_off, int k_off, int v_off,
     const float* __restrict__ head_decay, const float* __restrict__ z, long long z_stride, float inv_tau,
     float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ req_slots,
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(256) void la_scan_kernel(
 
   for (int t0 = begin; t0 < end; t0 += LA_TB) {
     const int nt = end - t0 < LA_TB ? end - t0 : LA_TB;
-    for (int idx = tid; idx < nt * DG; idx += 256) {
+    for (int idx = tid; idx < nt * DG; idx += LA_THREADS) {
       const int t = idx / DG, d = idx % DG;
       const TP* row = proj + (size_t)(t0 + t) * proj_stride + (size_t)head * LA_DIM + d0 + d;
       qs[t][d] = la_act(ldf<TP>(row + q_off), act) * q_scale;
@@ -94,11 +96,15 @@ __global__ __launch_bounds__(256) void la_scan_kernel(
       }
     }
     __syncthreads();
-    for (int idx = tid; idx < nt * 64; idx += 256) {
+    for (int idx = tid; idx < nt * 64; idx += LA_THREADS) {
       const int t = idx >> 6, l = idx & 63;
       const int c = vtile * 64 + l;
-      if (c < vdim)
-        out[((size_t)(t0 + t) * H + head) * vdim + c] = ((po[t][0][l] + po[t][1][l]) + po[t][2][l]) + po[t][3][l];
+      if (c < vdim) {
+        float sum = po[t][0][l];
+#pragma unroll
+        for (int w = 1; w < LA_WAVES; ++w) sum += po[t][w][l];
+        out[((size_t)(t0 + t) * H + head) * vdim + c] = sum;
+      }
     }
     __syncthreads();
   }
@@ -244,7 +250,7 @@ extern "C" int qvl_la_scan(const void* proj, long long proj_stride, int q_off, i
   if (H > 65535 || R > 65535) return QVL_ERR_LIMIT;
   const dim3 grid(((vdim + 63) / 64) * groups, H, R);
 #define LAUNCH(TP, CH, G)                                                                                           \
-  hipLaunchKernelGGL((la_scan_kernel<TP, CH, G>), grid, dim3(256), 0, stream, (const TP*)proj, proj_stride, q_off,   \
+  hipLaunchKernelGGL((la_scan_kernel<TP, CH, G>), grid, dim3(LA_THREADS), 0, stream, (const TP*)proj, proj_stride, q_off,   \
                      k_off, v_off, (const float*)head_decay, (const float*)z, z_stride, inv_tau, (float*)state,      \
                      (const int*)cu_q, (const int*)req_slots, (float*)out, out_slab, H, vdim, act, q_scale)
 #define BY_GROUPS(TP, CH)                                                                                           \

@@ -46,7 +46,7 @@ def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
     _dev(proj, state, cu_q, req_slots, head_decay, z)
     h, d, v = int(num_heads), int(dim), int(vdim)
     n = proj.shape[0]
-    _need(d % 4 == 0 and 4 <= d <= MAX_KEY_SIZE, f"key sizes in steps of 4 up to {MAX_KEY_SIZE} are built")
+    _need(1 <= d <= MAX_KEY_SIZE, f"key sizes up to {MAX_KEY_SIZE} are built")
     _need(proj.dim() == 2 and proj.stride(1) == 1, "proj must be [N, cols] with contiguous rows")
     for off, width in ((q_off, h * d), (k_off, h * d), (v_off, h * v)):
         _need(0 <= off and off + width <= proj.shape[1], "q, k or v columns lie outside proj")
@@ -65,7 +65,8 @@ def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
         _need(z.dtype == torch.float32 and z.shape == (n, h * d) and z.stride(1) == 1, "z must be float32 [N, heads dim]")
         _need(tau > 0, "tau must be positive")
         zstride = z.stride(0)
-    _need(groups in (1, 2, 4, 8) and d % (4 * groups) == 0, "groups must be 1, 2, 4 or 8 and divide a quarter of the key size")
+    _need(groups == 1 or (groups in (2, 4, 8) and d % (4 * groups) == 0),
+          "groups must be 1, 2, 4 or 8 and divide a quarter of the key size")
     if out is None:
         out = torch.empty((groups, n, h * v), dtype=torch.float32, device=proj.device)
     _need(out.dtype == torch.float32 and out.shape == (groups, n, h * v) and out.is_contiguous() and out.is_cuda,

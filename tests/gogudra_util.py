@@ -63,6 +63,15 @@ NO_PAGES = config(40, 64, [
 ], eps=1e-6, softcap=4.0)
 
 
+# Odd everything: a width that eight does not divide, key sizes that four (or two) does not divide, value
+# sizes below a wave, an odd inner size of the decay projection, an odd vocabulary.
+ODD = config(50, 101, [
+    gla_layer(3, 6, 7, 2.0, dense(30, 1.2)),
+    lightning_layer(2, 5, 9, [0.9, 0.6]),
+    attention_layer(3, 3, 10, 6, base=77.0, scale=0.4, mlp=dense(22, 2.0)),
+], eps=1e-5, softcap=6.0)
+
+
 def tensor_shapes(cfg: dict, rank: int = 6) -> Dict[str, tuple]:
     w = cfg["width"]
     shapes = {"embed": (cfg["vocab"], w), "final.norm": (w,)}

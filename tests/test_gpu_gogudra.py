@@ -20,7 +20,8 @@ F64 = torch.float64
 def folders(tmp_path_factory):
     out = {}
     for name, cfg, seed, rank, sharp in (("mixed", gu.MIXED, 11, 6, 1.0), ("sharp", gu.MIXED, 12, 6, 6.0),
-                                         ("ones", gu.ONES, 13, 3, 2.0), ("no_pages", gu.NO_PAGES, 14, 10, 1.0)):
+                                         ("ones", gu.ONES, 13, 3, 2.0), ("no_pages", gu.NO_PAGES, 14, 10, 1.0),
+                                         ("odd", gu.ODD, 15, 5, 1.0)):
         out[name] = gu.write_model(str(tmp_path_factory.mktemp(name)), cfg, seed, rank, sharp)
     return out
 
@@ -246,6 +247,20 @@ def test_sharpening_matters(folders):
     whole = _oracle(folders["sharp"], toks)[-1:]
     cut = _oracle(folders["sharp"], toks[200:])[-1:]
     assert _rel(cut, whole) > 0.05
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_odd_sizes_and_a_long_prompt(dtype, folders):
+    """Sizes that no vector width divides, in a prompt long enough for the chunked recurrence, whole and in portions."""
+    folder = folders["odd"]
+    reqs = {"o": random_tokens(150, gu.ODD["vocab"], 80), "p": random_tokens(3, gu.ODD["vocab"], 81)}
+    want = {rid: _oracle(folder, toks) for rid, toks in reqs.items()}
+    bound = 2e-5 if dtype == "float32" else 3 * max(
+        _rel(_oracle(folder, toks, plain.to_bfloat16_and_back), want[rid]) for rid, toks in reqs.items())
+    for steps in (whole_trace(reqs), portion_trace(reqs, (130, 2, 5, 13))):
+        got = run_steps(_replayer(folder, dtype, 256), steps)
+        for rid, toks in reqs.items():
+            assert _rel(_rows(got, rid, len(toks)), want[rid]) < bound, (dtype, rid)
 
 
 def test_long_decoding(folders):
