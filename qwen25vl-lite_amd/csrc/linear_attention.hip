@@ -26,7 +26,7 @@
 // waves of a block: four share the rows of S where the key size divides by four, else two or one
 #define LA_WAVES (LA_DIM % 4 == 0 ? 4 : (LA_DIM % 2 == 0 ? 2 : 1))
 #define LA_THREADS (64 * LA_WAVES)
-#define LA_TB (LA_DIM > 128 ? 8 : 16)
+#define LA_TB (LA_DIM > 256 ? 4 : (LA_DIM > 128 ? 8 : 16))
 
 
 __device__ __forceinline__ float la_act(float z, int act) { return act ? z / (1.0f + expf(-z)) : z; }
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(LA_THREADS) void la_scan_kernel(
 // stay as they are), last [chunks, H, LA_DIM].  The chunk's tokens are cut into LA_PARTS ranges; a thread
 // sums the logarithms of its channel's decays over its range, learns through LDS what the ranges before
 // it add up to, and walks its range again to write q_t * P_t.
-#define LA_PARTS (LA_DIM <= 64 ? 8 : (LA_DIM <= 128 ? 4 : 2))
+#define LA_PARTS (LA_DIM <= 64 ? 8 : (LA_DIM <= 128 ? 4 : (LA_DIM <= 256 ? 2 : 1)))
 
 template <typename TP, bool CHANNEL_DECAY>
 __global__ void la_prefix_kernel(const TP* __restrict__ proj, long long proj_stride, int q_off,

@@ -21,8 +21,8 @@ LIBRARIES = [
     ("peaks", {}),
     ("gated", {}),
     # the linear-attention kernels are compiled per key size (the sizes the tests and the benchmark
-    # use; any other size up to 256 is compiled at its first use)
-    *[("linear_attention", {"LA_DIM": d}) for d in (5, 6, 8, 12, 16, 20, 32, 64, 128)],
+    # use; any other size up to 512 is compiled at its first use)
+    *[("linear_attention", {"LA_DIM": d}) for d in (5, 6, 8, 12, 16, 20, 32, 64, 128, 320)],
     # the matrix-core attention is compiled per head size; these are the sizes the tests and the
     # benchmark use, any other multiple of 16 is compiled at its first use
     ("attention_mfma", {"HD": 128}),

@@ -19,7 +19,7 @@ from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
 __all__ = ["decayed_scan", "scan_groups", "chunked_scan", "plan_chunks", "ChunkPlan", "MAX_KEY_SIZE", "CHUNK"]
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
-MAX_KEY_SIZE = 256
+MAX_KEY_SIZE = 512
 LONG_RUN = 64
 BLOCKS_PER_CU = 2
 MIN_ROWS = 4

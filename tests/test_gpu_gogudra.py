@@ -330,6 +330,27 @@ def test_scan_cut_into_groups_of_key_channels():
             assert st[1].abs().max() == 0
 
 
+def test_a_large_key_size():
+    """Keys of 320 channels: fewer tokens are staged at a time and the decays' prefix is not cut."""
+    from qwen25vl_lite_amd.ops.linear_attention import chunked_scan, decayed_scan, plan_chunks
+    torch.manual_seed(12)
+    n, h, d, v = 130, 1, 320, 24
+    proj = (0.2 * torch.randn(n, 2 * h * d + h * v)).cuda()
+    z = (3 + torch.randn(n, h * d)).cuda()
+    cu = torch.tensor([0, n], dtype=torch.int32).cuda()
+    slots = torch.tensor([0], dtype=torch.int32).cuda()
+    s1 = torch.zeros(1, h, d, v).cuda()
+    got = decayed_scan(proj, 0, h * d, 2 * h * d, h, d, v, s1, cu, slots, z=z, tau=1.5).sum(0).cpu().double()
+    p = proj.cpu().double()
+    decay = torch.exp(torch.nn.functional.logsigmoid(z.cpu().double()) / 1.5)
+    want, s_end = plain.decayed_outer_product_scan(p[:, :d], p[:, d:2 * d], p[:, 2 * d:], decay)
+    assert torch.allclose(got, want, atol=2e-5 * want.abs().max().item())
+    assert torch.allclose(s1[0, 0].cpu().double(), s_end, atol=2e-5 * s_end.abs().max().item())
+    s2 = torch.zeros(1, h, d, v).cuda()
+    cut = chunked_scan(proj, 0, h * d, 2 * h * d, h, d, v, s2, plan_chunks([0, n], "cuda:0"), slots, z=z, tau=1.5)
+    assert torch.allclose(cut.sum(0).cpu().double(), want, atol=2e-5 * want.abs().max().item())
+
+
 @pytest.mark.parametrize("channel", [False, True])
 def test_long_runs_scanned_in_chunks(channel):
     """Runs cut into chunks that are scanned side by side and stitched through the carried state: the
