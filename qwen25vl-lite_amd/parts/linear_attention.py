@@ -131,9 +131,8 @@ class LinearAttention(Mixer):
         z = None
         if self.decay_kind == "channel":
             at = 2 * hk + 2 * hv
-            low = proj[:, at:at + self.rank]         # a few columns: copied to rows of their own
-            z = linear(low.contiguous(), self.w_a2, self.b_a2,
-                       out_dtype=torch.float32)
+            low = proj[:, at:at + self.rank].contiguous()      # a few columns: copied to rows of their own
+            z = linear(low, self.w_a2, self.b_a2, out_dtype=torch.float32)
         how = dict(head_decay=self.head_decay, z=z, tau=self.tau, silu=self.activation == "silu", q_scale=self.q_scale)
         if step.max_q_len >= CHUNKED_FROM and len(step.cu_q_host) == step.num_reqs + 1:
             # long runs (never a captured decode step): in chunks side by side; the plan is the step's, shared by layers
