@@ -138,7 +138,7 @@ class CacheManager:
     def commit(self, req_id, num_tokens: int) -> None:
         """Tokens ``[0, num_tokens)`` are now in the cache.  A windowed group gives back the
         pages no later token can see: the next query sits at index ``num_tokens`` and sees keys
-        from ``num_tokens - window + 1`` on."""
+        from ``num_tokens - window + 1`` on, and the group's first ``keep_first`` keys."""
         rp = self.requests[req_id]
         if num_tokens < rp.num_tokens:
             raise ValueError("a request's cached length cannot shrink")
@@ -146,10 +146,12 @@ class CacheManager:
         self.records.num_tokens[rp.slot] = num_tokens
         for g, table in enumerate(rp.tables):
             first = min(self._first_needed_page(g, num_tokens), len(table))
-            gone = [p for p in table[:first] if p >= 0]
+            # pages that hold any of the first keep_first tokens stay: every later token reads them
+            kept = (self.groups[g].need.keep_first + self.page_size - 1) // self.page_size
+            gone = [p for p in table[kept:first] if p >= 0]
             if gone:
                 self.pools[g].free(gone)
-                for i in range(first):
+                for i in range(kept, first):
                     table[i] = -1
 
     def table(self, req_id, group: int) -> List[int]:

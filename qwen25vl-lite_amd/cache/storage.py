@@ -13,7 +13,7 @@ __all__ = ["KVStorage"]
 
 class KVStorage:
     """Keys and values of every group: per group ``k`` of ``[layers, pages, nkv, page_size, hd]``
-    and ``v`` of ``[layers, pages, nkv, hd, page_size]``.  One kv head's keys of a page are a
+    and ``v`` of ``[layers, pages, nkv, vd, page_size]`` (``vd`` the value size, ``hd`` unless the group says otherwise).  One kv head's keys of a page are a
     contiguous ``page_size x hd`` tile; values are kept transposed so that the matrix-core
     kernels read eight consecutive keys of one channel with a single 16-byte load.
     The logical content is the reference's ``[layers, blocks, block_size, kv_heads, head_dim]``
@@ -26,9 +26,9 @@ class KVStorage:
         self.k: List[torch.Tensor] = []
         self.v: List[torch.Tensor] = []
         for g in groups:
-            nkv, hd = g.need.num_kv_heads, g.need.head_dim
+            nkv, hd, vd = g.need.num_kv_heads, g.need.head_dim, g.need.v_dim
             self.k.append(torch.zeros((g.num_layers, num_pages, nkv, page_size, hd), dtype=dtype, device=device))
-            self.v.append(torch.zeros((g.num_layers, num_pages, nkv, hd, page_size), dtype=dtype, device=device))
+            self.v.append(torch.zeros((g.num_layers, num_pages, nkv, vd, page_size), dtype=dtype, device=device))
 
     def copy_pages(self, group: int, src: Sequence[int], dst: Sequence[int]) -> None:
         """Keys and values of pages ``src`` into pages ``dst`` of a group, in all of its layers

@@ -317,94 +317,202 @@ extern "C" int qvl_head_gate(void* o, const void* gate, long long gate_stride, i
 }
 
 // ---------------------------------------------------------------------------------------
-// Queries and keys of attention with a per-head norm before the rotation:
-//   x [N, stride] float32: nq query heads, then nkv key heads (then nkv value heads unless the
-//   values are the keys as projected: `v_from_k`).
+// Queries and keys of attention with a per-head norm before or after the rotation:
+//   x [N, stride] float32: nq query heads and nkv key heads of hd channels, then nkv value heads of
+//   vd channels (none if the values are the keys as projected: `v_from_k`).  `bias` (or null) is
+//   added to every column first.
 //   head vector a -> a / sqrt(mean(a^2) + eps) * nw (nw = qw for query heads, kw for key heads; a
-//   null weight skips the norm) -> rotation of the first 2 rot_half channels by the angles whose
+//   null weight is a gain of one) -> rotation of the first 2 rot_half channels by the angles whose
 //   cosines and sines are cs[n, f]: pair (2f, 2f+1) if `interleaved`, else (f, f + rot_half).
+//   norm_mode 0: no norm; 1: the norm comes before the rotation; 2: after it.
 //   Queries go to q_out [N, nq hd]; keys into k_cache [pages, nkv, ps, hd] at slots[n]; values
-//   (the key head before norm and rotation, or the value head) into v_cache [pages, nkv, hd, ps].
-// One wave per (token, head); a block holds 4 of them.  hd <= 512.
+//   (the key head before norm and rotation, or the value head) into v_cache [pages, nkv, vd, ps].
+// One wave per (token, head); a block holds 4 of them.  hd, vd <= 512.
 // ---------------------------------------------------------------------------------------
 #define QKN_MAX_HD 512
 
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
-    const float* __restrict__ x, long long x_stride, const float* __restrict__ qw, const float* __restrict__ kw,
-    const float2* __restrict__ cs, const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, int N, int nq, int nkv, int hd, int rot_half, int ps, float eps, int interleaved,
-    int v_from_k, int write_kv) {
+    const float* __restrict__ x, long long x_stride, const float* __restrict__ bias, const float* __restrict__ qw,
+    const float* __restrict__ kw, const float2* __restrict__ cs, const int* __restrict__ slots, T* __restrict__ q_out,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int N, int nq, int nkv, int hd, int vd, int rot_half, int ps,
+    float eps, int interleaved, int v_from_k, int write_kv, int norm_mode) {
   __shared__ float buf[4][QKN_MAX_HD];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int heads = nq + (write_kv ? (v_from_k ? nkv : 2 * nkv) : 0);
   const long long item = (long long)blockIdx.x * 4 + wave;
   if (item >= (long long)N * heads) return;
   const int n = (int)(item / heads), head = (int)(item % heads);
-  const float* a = x + (size_t)n * x_stride + (size_t)head * hd;
+  const int kind = head < nq ? 0 : (head < nq + nkv ? 1 : 2);   // query, key, value head
+  const size_t col = kind == 2 ? (size_t)(nq + nkv) * hd + (size_t)(head - nq - nkv) * vd : (size_t)head * hd;
+  const float* a = x + (size_t)n * x_stride + col;
+  const float* b = bias ? bias + col : nullptr;
   float* mine = buf[wave];
   const int slot = (head >= nq && write_kv) ? slots[n] : -1;
-  const int kind = head < nq ? 0 : (head < nq + nkv ? 1 : 2);   // query, key, value head
   if (kind != 0 && slot < 0) return;                            // a padding row writes nowhere
   const size_t page = slot >= 0 ? (size_t)(slot / ps) : 0;
   const int in_page = slot >= 0 ? slot % ps : 0;
   if (kind == 2) {
     const int kvh = head - nq - nkv;
-    T* vrow = v_cache + ((page * nkv + kvh) * hd) * (size_t)ps + in_page;
-    for (int c = lane; c < hd; c += 64) stf<T>(vrow + (size_t)c * ps, a[c]);
+    T* vrow = v_cache + ((page * nkv + kvh) * vd) * (size_t)ps + in_page;
+    for (int c = lane; c < vd; c += 64) stf<T>(vrow + (size_t)c * ps, a[c] + (b ? b[c] : 0.f));
     return;
   }
   float ss = 0.f;
   for (int c = lane; c < hd; c += 64) {
-    const float v = a[c];
+    const float v = a[c] + (b ? b[c] : 0.f);
     mine[c] = v;
     ss += v * v;
   }
   const float* nw = kind == 0 ? qw : kw;
-  const float rs = nw ? 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps) : 1.0f;
   if (kind == 1 && v_from_k) {
     const int kvh = head - nq;
-    T* vrow = v_cache + ((page * nkv + kvh) * hd) * (size_t)ps + in_page;
+    T* vrow = v_cache + ((page * nkv + kvh) * vd) * (size_t)ps + in_page;
     for (int c = lane; c < hd; c += 64) stf<T>(vrow + (size_t)c * ps, mine[c]);
   }
-  if (nw)
-    for (int c = lane; c < hd; c += 64) mine[c] = (mine[c] * rs) * nw[c];
+  if (norm_mode == 1) {
+    const float rs = 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps);
+    for (int c = lane; c < hd; c += 64) mine[c] = nw ? (mine[c] * rs) * nw[c] : mine[c] * rs;
+  }
   __builtin_amdgcn_wave_barrier();
   T* dst = kind == 0 ? q_out + ((size_t)n * nq + head) * hd
                      : k_cache + ((page * nkv + (head - nq)) * ps + in_page) * (size_t)hd;
   const float2* csn = cs + (size_t)n * rot_half;
-  for (int c = lane; c < hd; c += 64) {
-    float v = mine[c];
-    if (c < 2 * rot_half) {
-      int f, partner;
-      bool first;
-      if (interleaved) { f = c >> 1; first = !(c & 1); partner = c ^ 1; }
-      else { first = c < rot_half; f = first ? c : c - rot_half; partner = first ? c + rot_half : c - rot_half; }
-      const float2 t = csn[f];
-      const float p = mine[partner];
-      v = first ? v * t.x - p * t.y : v * t.x + p * t.y;
+  float turned[QKN_MAX_HD / 64];
+  float ss2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < QKN_MAX_HD / 64; ++i) {
+    const int c = lane + 64 * i;
+    float v = 0.f;
+    if (c < hd) {
+      v = mine[c];
+      if (c < 2 * rot_half) {
+        int f, partner;
+        bool first;
+        if (interleaved) { f = c >> 1; first = !(c & 1); partner = c ^ 1; }
+        else { first = c < rot_half; f = first ? c : c - rot_half; partner = first ? c + rot_half : c - rot_half; }
+        const float2 t = csn[f];
+        const float p = mine[partner];
+        v = first ? v * t.x - p * t.y : v * t.x + p * t.y;
+      }
     }
-    stf<T>(dst + c, v);
+    turned[i] = v;
+    ss2 += v * v;
+  }
+  const float rs2 = norm_mode == 2 ? 1.0f / sqrtf(wave_sum(ss2) / (float)hd + eps) : 1.0f;
+#pragma unroll
+  for (int i = 0; i < QKN_MAX_HD / 64; ++i) {
+    const int c = lane + 64 * i;
+    if (c < hd) {
+      float v = turned[i];
+      if (norm_mode == 2) v = nw ? (v * rs2) * nw[c] : v * rs2;
+      stf<T>(dst + c, v);
+    }
   }
 }
 
-extern "C" int qvl_qk_norm_rope_write(const void* x, long long x_stride, const void* qw, const void* kw, const void* cs,
-                                      const void* slots, void* q_out, void* k_cache, void* v_cache, int N, int nq,
-                                      int nkv, int hd, int rot_half, int ps, float eps, int interleaved, int v_from_k,
-                                      int write_kv, int dtype, hipStream_t stream) {
+extern "C" int qvl_qk_norm_rope_write(const void* x, long long x_stride, const void* bias, const void* qw,
+                                      const void* kw, const void* cs, const void* slots, void* q_out, void* k_cache,
+                                      void* v_cache, int N, int nq, int nkv, int hd, int vd, int rot_half, int ps,
+                                      float eps, int interleaved, int v_from_k, int write_kv, int norm_mode, int dtype,
+                                      hipStream_t stream) {
   if (N <= 0) return QVL_OK;
-  if (nq <= 0 || nkv < 0 || hd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0) return QVL_ERR_SHAPE;
+  if (nq <= 0 || nkv < 0 || hd <= 0 || vd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0) return QVL_ERR_SHAPE;
   if (write_kv && (!slots || !k_cache || !v_cache || nkv <= 0)) return QVL_ERR_SHAPE;
-  if (hd > QKN_MAX_HD) return QVL_ERR_LIMIT;
+  if (norm_mode < 0 || norm_mode > 2 || (v_from_k && vd != hd)) return QVL_ERR_SHAPE;
+  if (hd > QKN_MAX_HD || vd > QKN_MAX_HD) return QVL_ERR_LIMIT;
   const int heads = nq + (write_kv ? (v_from_k ? nkv : 2 * nkv) : 0);
   const long long items = (long long)N * heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
 #define LAUNCH(T)                                                                                                  \
   hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(blocks), dim3(256), 0, stream, (const float*)x, x_stride,   \
-                     (const float*)qw, (const float*)kw, (const float2*)cs, (const int*)slots, (T*)q_out,          \
-                     (T*)k_cache, (T*)v_cache, N, nq, nkv, hd, rot_half, ps, eps, interleaved, v_from_k, write_kv)
+                     (const float*)bias, (const float*)qw, (const float*)kw, (const float2*)cs, (const int*)slots, \
+                     (T*)q_out, (T*)k_cache, (T*)v_cache, N, nq, nkv, hd, vd, rot_half, ps, eps, interleaved,      \
+                     v_from_k, write_kv, norm_mode)
   if (dtype == 0) LAUNCH(float);
   else if (dtype == 1) LAUNCH(bf16_t);
+  else return QVL_ERR_DTYPE;
+#undef LAUNCH
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// The sum of a residual stream whose sublayers are normed on their way in:
+//   h[n, :] += factor * (y[n, :] / sqrt(mean(y[n]^2) + eps_y)) * gain + vec
+// (y float32 or bfloat16, or float32 slabs added in order; a null gain adds y as it is; a null y
+// adds nothing; vec, or null, is one vector for every row), and, if `out` is given, the next norm
+//   out[m, :] = h[n, :] / sqrt(mean(h[n]^2) + eps) * w
+// With `rows`, n = rows[m] and h is only read (the sum is formed for the rows asked for).
+// One block per row; a thread keeps its values of the row in registers between the passes.
+// ---------------------------------------------------------------------------------------
+#define SN_VPT 16
+
+template <typename TY, typename TO>
+__global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict__ y, int nslabs, long long slab_stride,
+                                     const float* __restrict__ gain, float eps_y, float factor,
+                                     const float* __restrict__ vec, const float* __restrict__ w, float eps,
+                                     TO* __restrict__ out, const int* __restrict__ rows, int H) {
+  __shared__ float red[17];
+  const int m = blockIdx.x, n = rows ? rows[m] : m;
+  float* hr = h + (size_t)n * H;
+  float val[SN_VPT];
+  float rs = 1.0f;
+  if (y) {
+    const TY* yr = y + (size_t)n * H;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < SN_VPT; ++i) {
+      const int c = threadIdx.x + i * blockDim.x;
+      float v = 0.f;
+      if (c < H) {
+        v = ldf<TY>(yr + c);
+        for (int s = 1; s < nslabs; ++s) v += ldf<TY>(yr + (size_t)s * slab_stride + c);
+      }
+      val[i] = v;
+      ss += v * v;
+    }
+    if (gain) rs = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps_y);
+  }
+  float ss2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < SN_VPT; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    float v = 0.f;
+    if (c < H) {
+      v = hr[c];
+      if (y) v += gain ? factor * ((val[i] * rs) * gain[c]) : val[i];
+      if (vec) v += vec[c];
+      if (!rows && (y || vec)) hr[c] = v;
+    }
+    val[i] = v;
+    ss2 += v * v;
+  }
+  if (!out) return;
+  const float rs2 = 1.0f / sqrtf(block_sum(ss2, red) / (float)H + eps);
+  TO* o = out + (size_t)m * H;
+#pragma unroll
+  for (int i = 0; i < SN_VPT; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < H) stf<TO>(o + c, (val[i] * rs2) * w[c]);
+  }
+}
+
+extern "C" int qvl_sandwich_norm(void* h, const void* y, int y_dtype, int nslabs, long long slab_stride, const void* gain,
+                                 float eps_y, float factor, const void* vec, const void* w, float eps, void* out,
+                                 int out_dtype, const void* rows, int M, int H, hipStream_t stream) {
+  if (M <= 0) return QVL_OK;
+  if (H <= 0 || nslabs < 1 || (nslabs > 1 && y_dtype != 0) || (out && !w)) return QVL_ERR_SHAPE;
+  if (H > 1024 * SN_VPT) return QVL_ERR_LIMIT;
+  int threads = (H + SN_VPT - 1) / SN_VPT;
+  threads = threads <= 256 ? 256 : (threads + 63) / 64 * 64;
+#define LAUNCH(TY, TO)                                                                                              \
+  hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO>), dim3(M), dim3(threads), 0, stream, (float*)h, (const TY*)y,    \
+                     nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec, (const float*)w,    \
+                     eps, (TO*)out, (const int*)rows, H)
+  if (y_dtype == 0 && out_dtype == 0) LAUNCH(float, float);
+  else if (y_dtype == 0 && out_dtype == 1) LAUNCH(float, bf16_t);
+  else if (y_dtype == 1 && out_dtype == 1) LAUNCH(bf16_t, bf16_t);
+  else if (y_dtype == 1 && out_dtype == 0) LAUNCH(bf16_t, float);
   else return QVL_ERR_DTYPE;
 #undef LAUNCH
   return qvl_launch_status();

@@ -1,0 +1,355 @@
+// A feed-forward made of many small experts, of which every token uses a few:
+//   route    scores of the router's logits, the choice of experts within the best groups, weights
+//   sort     the (token, choice) pairs listed by expert
+//   products x W_e^T for every expert's pairs: gate|up with the gated activation, then down
+//   combine  the weighted sum of a token's experts, plus what a shared expert gave
+// float32 and bfloat16 storage; scores, weights and sums are float32.  A pair is p = token * top + choice.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// ---------------------------------------------------------------------------------------
+// Router.  z [N, E] float32 logits.  s = sigmoid(z) (score_fn 0) or softmax(z) over the experts
+// (score_fn 1).  The experts form `groups` equal groups of neighbours; a group's score is the sum of
+// its two largest s (of its one, if it has one); only experts of the `keep` best groups can be
+// chosen; the `top` largest s among those are the choice (ties: the lower index).  Weights: the
+// chosen s divided by (their sum + floor) if `normalize`, times `scale`.
+// One wave per token; E <= 512, groups <= 64.
+// ---------------------------------------------------------------------------------------
+#define MOE_MAX_E 512
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, int* __restrict__ ids,
+                                                        float* __restrict__ wts, int N, int E, int top, int groups,
+                                                        int keep, float scale, int score_fn, int normalize,
+                                                        float floor_) {
+  __shared__ float s_all[4][MOE_MAX_E];
+  __shared__ float g_all[4][64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + wave;
+  if (n >= N) return;
+  float* s = s_all[wave];
+  float* gs = g_all[wave];
+  const float* zr = z + (size_t)n * E;
+  if (score_fn == 1) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float v = expf(zr[e] - mx);
+      s[e] = v;
+      sum += v;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) s[e] = s[e] / sum;
+  } else {
+    for (int e = lane; e < E; e += 64) s[e] = sigmoid_f(zr[e]);
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int per = E / groups;
+  if (lane < groups) {
+    float a = -INFINITY, b = -INFINITY;   // the two largest
+    for (int i = 0; i < per; ++i) {
+      const float v = s[lane * per + i];
+      if (v > a) { b = a; a = v; }
+      else if (v > b) b = v;
+    }
+    gs[lane] = per > 1 ? a + b : a;
+  }
+  __builtin_amdgcn_wave_barrier();
+  bool allowed_group = false;
+  if (lane < groups) {
+    int ahead = 0;
+    const float mine = gs[lane];
+    for (int g = 0; g < groups; ++g) ahead += (gs[g] > mine || (gs[g] == mine && g < lane)) ? 1 : 0;
+    allowed_group = ahead < keep;
+  }
+  const unsigned long long allowed = __ballot(allowed_group);
+  // this lane's experts: e = lane + 64 i; a score of -1 can never be chosen before an allowed one
+  float cand[MOE_MAX_E / 64];
+#pragma unroll
+  for (int i = 0; i < MOE_MAX_E / 64; ++i) {
+    const int e = lane + 64 * i;
+    cand[i] = (e < E && ((allowed >> (e / per)) & 1ull)) ? s[e] : -1.0f;
+  }
+  float total = 0.f;
+  float my_w = 0.f;   // lane t keeps the weight of choice t (top <= 64)
+  int my_id = 0;
+  for (int t = 0; t < top; ++t) {
+    float best = -2.0f;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_E / 64; ++i)
+      if (cand[i] > best) { best = cand[i]; at = lane + 64 * i; }
+    // the wave's best: larger score first, then the lower index
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, QVL_WAVE);
+      const int oa = __shfl_xor(at, o, QVL_WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if ((at & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < MOE_MAX_E / 64; ++i)
+        if (at == lane + 64 * i) cand[i] = -3.0f;
+    }
+    total += best;
+    if (lane == t) { my_w = best; my_id = at; }
+  }
+  if (lane < top) {
+    const float w = normalize ? my_w / (total + floor_) : my_w;
+    ids[(size_t)n * top + lane] = my_id;
+    wts[(size_t)n * top + lane] = w * scale;
+  }
+}
+
+extern "C" int qvl_moe_route(const void* z, void* ids, void* wts, int N, int E, int top, int groups, int keep,
+                             float scale, int score_fn, int normalize, float floor_, hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (E <= 0 || top <= 0 || groups <= 0 || keep <= 0 || keep > groups || E % groups || top > keep * (E / groups))
+    return QVL_ERR_SHAPE;
+  if (E > MOE_MAX_E || groups > 64 || top > 64) return QVL_ERR_LIMIT;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((N + 3) / 4), dim3(256), 0, stream, (const float*)z, (int*)ids, (float*)wts, N,
+                     E, top, groups, keep, scale, score_fn, normalize, floor_);
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Pairs listed by expert: offsets[e] .. offsets[e + 1] of `sorted` hold the pairs that chose expert
+// e (in no fixed order: a pair's row of a product does not depend on its neighbours).  One block.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int* __restrict__ sorted,
+                                                        int* __restrict__ offsets, int P, int E) {
+  __shared__ int count[MOE_MAX_E + 1];
+  __shared__ int start[MOE_MAX_E + 1];
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = at;
+      at += count[e];
+    }
+    start[E] = at;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) {
+    offsets[e] = start[e];
+    count[e] = 0;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < E) sorted[start[e] + atomicAdd(&count[e], 1)] = p;
+  }
+}
+
+extern "C" int qvl_moe_sort(const void* ids, void* sorted, void* offsets, int P, int E, hipStream_t stream) {
+  if (P <= 0) return QVL_OK;
+  if (E <= 0) return QVL_ERR_SHAPE;
+  if (E > MOE_MAX_E) return QVL_ERR_LIMIT;
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, (const int*)ids, (int*)sorted, (int*)offsets, P, E);
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// The experts' products.  For the pair p at place i of `sorted` (expert e by `offsets`):
+//   in = x[p / div, :]            (div = top for the first product, whose rows are tokens; 1 for the second)
+//   plain:  out[p, c] = in . W[e, c, :]
+//   gated:  g = min(in . W[e, c, :], limit), u = clamp(in . W[e, R + c, :], -limit, limit)  (no clamps if limit <= 0)
+//           out[p, c] = g * sigmoid(alpha g) * (u + shift)            (W[e] holds R gate rows, then R up rows)
+// Any sizes and both storage types: one wave per output value, lanes split K (the sum's order is fixed).
+// ---------------------------------------------------------------------------------------
+struct ExpertArgs {
+  const void* x;
+  long long ldx;
+  const void* w;        // [E, rows_w, K]
+  const int* sorted;
+  const int* offsets;
+  void* out;            // [P, R]
+  int P, E, R, K, div, gated;
+  float alpha, limit, shift;
+};
+
+__device__ __forceinline__ float gated_value(float g, float u, float alpha, float limit, float shift) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  return g * sigmoid_f(alpha * g) * (u + shift);
+}
+
+__device__ __forceinline__ int expert_of(const int* offsets, int E, int i) {
+  int e = 0;
+  while (e + 1 < E && offsets[e + 1] <= i) ++e;
+  return e;
+}
+
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void moe_rows_kernel(ExpertArgs a) {
+  const int i = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int e = expert_of(a.offsets, a.E, i);
+  const int p = a.sorted[i];
+  const T* xr = (const T*)a.x + (size_t)(p / a.div) * a.ldx;
+  const int rows_w = a.gated ? 2 * a.R : a.R;
+  const T* we = (const T*)a.w + (size_t)e * rows_w * a.K;
+  for (int c = blockIdx.y * 4 + wave; c < a.R; c += gridDim.y * 4) {
+    const T* wg = we + (size_t)c * a.K;
+    float g = 0.f, u = 0.f;
+    for (int k = lane; k < a.K; k += 64) g += ldf<T>(xr + k) * ldf<T>(wg + k);
+    g = wave_sum(g);
+    if (a.gated) {
+      const T* wu = we + (size_t)(a.R + c) * a.K;
+      for (int k = lane; k < a.K; k += 64) u += ldf<T>(xr + k) * ldf<T>(wu + k);
+      u = wave_sum(u);
+      g = gated_value(g, u, a.alpha, a.limit, a.shift);
+    }
+    if (lane == 0) stf<TO>((TO*)a.out + (size_t)p * a.R + c, g);
+  }
+}
+
+// bfloat16 on the matrix cores.  A block of four waves owns 16 MT pairs of one expert and 64 output
+// columns; a wave takes 16 of the columns (rows of W: the instruction's first operand, straight from
+// memory: nobody else in the block reads them) and all MT tiles of 16 pairs (rows of x: the second
+// operand).  K in steps of 32, a multiple of 8.  Which expert a block serves follows from the
+// offsets: tile t of the grid is the (t - tiles before e)-th tile of 16 MT pairs of expert e.
+template <int MT, typename TO>
+__global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  constexpr int TM = 16 * MT;
+  int tile = blockIdx.x, e = 0, first = 0, last = 0;
+  for (; e < a.E; ++e) {
+    first = a.offsets[e];
+    last = a.offsets[e + 1];
+    const int nt = (last - first + TM - 1) / TM;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (e >= a.E) return;
+  first += tile * TM;
+  const int c0 = (blockIdx.y * 4 + wave) * 16;     // this wave's output columns
+  if (c0 >= a.R) return;
+  const int rows_w = a.gated ? 2 * a.R : a.R;
+  const bf16_t* we = (const bf16_t*)a.w + (size_t)e * rows_w * a.K;
+  const bool col_ok = c0 + r < a.R;
+  const bf16_t* wg = we + (size_t)(col_ok ? c0 + r : 0) * a.K + 8 * lg;
+  const bf16_t* wu = wg + (size_t)a.R * a.K;
+  const bf16_t* xr[MT];
+  int pair[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int i = first + 16 * t + r;
+    pair[t] = i < last ? a.sorted[i] : -1;
+    xr[t] = (const bf16_t*)a.x + (size_t)(pair[t] < 0 ? 0 : pair[t] / a.div) * a.ldx + 8 * lg;
+  }
+  f32x4_t accg[MT], accu[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    accg[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    accu[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const bf16x8_t zero = __builtin_bit_cast(bf16x8_t, uint4{0u, 0u, 0u, 0u});
+  for (int k = 0; k < a.K; k += 32) {
+    const bool k_ok = k + 8 * lg < a.K;
+    const bf16x8_t fg = (k_ok && col_ok) ? *reinterpret_cast<const bf16x8_t*>(wg + k) : zero;
+    bf16x8_t fu = zero;
+    if (a.gated && k_ok && col_ok) fu = *reinterpret_cast<const bf16x8_t*>(wu + k);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const bf16x8_t fx = (k_ok && pair[t] >= 0) ? *reinterpret_cast<const bf16x8_t*>(xr[t] + k) : zero;
+      accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg, fx, accg[t], 0, 0, 0);
+      if (a.gated) accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu, fx, accu[t], 0, 0, 0);
+    }
+  }
+  // a lane holds, of tile t, pair r and columns c0 + 4 lg .. + 3
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (pair[t] < 0) continue;
+    TO* o = (TO*)a.out + (size_t)pair[t] * a.R + c0 + 4 * lg;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (c0 + 4 * lg + j >= a.R) break;
+      float v = accg[t][j];
+      if (a.gated) v = gated_value(v, accu[t][j], a.alpha, a.limit, a.shift);
+      stf<TO>(o + j, v);
+    }
+  }
+}
+
+// x_dtype / out_dtype: 0 float32, 1 bfloat16.  float32 operands write float32; bfloat16 operands
+// write either.  The matrix-core kernel runs for bfloat16 with K a multiple of 8 and rows of x on
+// 16-byte boundaries; `big_tiles` asks for tiles of 64 pairs instead of 16 (many pairs an expert).
+extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const void* w, const void* sorted,
+                               const void* offsets, void* out, int out_dtype, int P, int E, int R, int K, int div,
+                               int gated, float alpha, float limit, float shift, int big_tiles, hipStream_t stream) {
+  if (P <= 0) return QVL_OK;
+  if (E <= 0 || R <= 0 || K <= 0 || div <= 0 || ldx < K || !x || !w || !sorted || !offsets || !out) return QVL_ERR_SHAPE;
+  ExpertArgs a;
+  a.x = x; a.ldx = ldx; a.w = w; a.sorted = (const int*)sorted; a.offsets = (const int*)offsets; a.out = out;
+  a.P = P; a.E = E; a.R = R; a.K = K; a.div = div; a.gated = gated; a.alpha = alpha; a.limit = limit; a.shift = shift;
+  if (x_dtype == 1 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0) {
+    const int tm = big_tiles ? 64 : 16;
+    const int tiles = P / tm + (E < P ? E : P);
+    const dim3 grid(tiles, (R + 63) / 64);
+    if (grid.y > 65535) return QVL_ERR_LIMIT;
+    if (big_tiles && out_dtype == 1) hipLaunchKernelGGL((moe_mfma_kernel<4, bf16_t>), grid, dim3(256), 0, stream, a);
+    else if (big_tiles && out_dtype == 0) hipLaunchKernelGGL((moe_mfma_kernel<4, float>), grid, dim3(256), 0, stream, a);
+    else if (out_dtype == 1) hipLaunchKernelGGL((moe_mfma_kernel<1, bf16_t>), grid, dim3(256), 0, stream, a);
+    else if (out_dtype == 0) hipLaunchKernelGGL((moe_mfma_kernel<1, float>), grid, dim3(256), 0, stream, a);
+    else return QVL_ERR_DTYPE;
+    return qvl_launch_status();
+  }
+  int by = (R + 3) / 4;
+  if (by > 64) by = 64;
+  const dim3 grid(P, by);
+  if (x_dtype == 0 && out_dtype == 0) hipLaunchKernelGGL((moe_rows_kernel<float, float>), grid, dim3(256), 0, stream, a);
+  else if (x_dtype == 1 && out_dtype == 1) hipLaunchKernelGGL((moe_rows_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, stream, a);
+  else if (x_dtype == 1 && out_dtype == 0) hipLaunchKernelGGL((moe_rows_kernel<bf16_t, float>), grid, dim3(256), 0, stream, a);
+  else return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// out[n, :] = sum over k of wts[n, k] * y[n top + k, :], in the order of k, plus `extra[n, :]` (what
+// a shared expert gave: float32 or bfloat16, or float32 slabs added in order; null: nothing).
+// ---------------------------------------------------------------------------------------
+template <typename TY, typename TX>
+__global__ void moe_combine_kernel(const TY* __restrict__ y, const float* __restrict__ wts, const TX* __restrict__ extra,
+                                   int nslabs, long long slab_stride, float* __restrict__ out, int top, int H) {
+  const size_t n = blockIdx.x;
+  const float* wr = wts + n * top;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) v += wr[k] * ldf<TY>(y + (n * top + k) * (size_t)H + c);
+    if (extra) {
+      float x = ldf<TX>(extra + n * H + c);
+      for (int s = 1; s < nslabs; ++s) x += ldf<TX>(extra + (size_t)s * slab_stride + n * H + c);
+      v += x;
+    }
+    out[n * H + c] = v;
+  }
+}
+
+extern "C" int qvl_moe_combine(const void* y, int y_dtype, const void* wts, const void* extra, int extra_dtype,
+                               int nslabs, long long slab_stride, void* out, int N, int top, int H, hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (top <= 0 || H <= 0 || nslabs < 1 || (nslabs > 1 && extra_dtype != 0)) return QVL_ERR_SHAPE;
+#define LAUNCH(TY, TX)                                                                                         \
+  hipLaunchKernelGGL((moe_combine_kernel<TY, TX>), dim3(N), dim3(256), 0, stream, (const TY*)y, (const float*)wts, \
+                     (const TX*)extra, nslabs, slab_stride, (float*)out, top, H)
+  if (y_dtype == 0 && extra_dtype == 0) LAUNCH(float, float);
+  else if (y_dtype == 0 && extra_dtype == 1) LAUNCH(float, bf16_t);
+  else if (y_dtype == 1 && extra_dtype == 0) LAUNCH(bf16_t, float);
+  else if (y_dtype == 1 && extra_dtype == 1) LAUNCH(bf16_t, bf16_t);
+  else return QVL_ERR_DTYPE;
+#undef LAUNCH
+  return qvl_launch_status();
+}

@@ -39,6 +39,23 @@ def _mixers_of(block: Part, prefix: str = "") -> List[Tuple[str, Mixer]]:
     return found
 
 
+class PassVectors(Part):
+    """Vectors ``[rows, hidden]`` in float32, one of which a run entry may add to every token's residual sum."""
+
+    graph_safe = True
+
+    def __init__(self, rows: int, hidden: int, dtype, device):
+        super().__init__(dtype, device)
+        self.rows, self.hidden = int(rows), int(hidden)
+        self.weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.rows, self.hidden), "vector")}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+
 class DecoderModel:
     """Holds the parts and runs a step over them.  Tensors arrive through :meth:`load_part`."""
 
@@ -52,6 +69,15 @@ class DecoderModel:
         self.embedding = build_part("embedding", spec.embed or PartSpec("token_table", sizes), dtype, self.device)
         self.head_part = build_part("head", spec.head or PartSpec("linear", sizes), dtype, self.device)
         self._has_weights = False
+        self.pass_vectors: Optional[PassVectors] = None
+        if spec.pass_vectors_name is not None:
+            if not spec.pass_vectors_name.endswith(".weight") or spec.pass_vectors_rows <= 0:
+                raise ValueError("pass vectors are a tensor '<name>.weight' with at least one row")
+            self.pass_vectors = PassVectors(spec.pass_vectors_rows, spec.hidden_size, dtype, self.device)
+        for i, entry in enumerate(spec.run):
+            if entry.add_vector is not None and not (self.pass_vectors is not None
+                                                     and 0 <= entry.add_vector < spec.pass_vectors_rows):
+                raise ValueError(f"run entry {i} adds pass vector {entry.add_vector}, which the model does not have")
 
         # The run list: which cache layer and state every mixer of every entry owns.  The lists
         # below have one element per (run entry, mixer of its block), in run order ("places");
@@ -107,6 +133,8 @@ class DecoderModel:
 
         self.params: Dict[str, Tuple[Optional[Part], str, ParamSpec]] = {}
         _collect(self.embedding, _prefix_of(spec.embed_name), self.params)
+        if self.pass_vectors is not None:
+            _collect(self.pass_vectors, _prefix_of(spec.pass_vectors_name), self.params)
         for ls, block in zip(spec.layers, self.blocks):
             _collect(block, ls.prefix, self.params)
         _collect(self.final_norm, spec.final_norm_prefix, self.params)
@@ -122,6 +150,7 @@ class DecoderModel:
         def safe(part) -> bool:
             return part.graph_safe and all(safe(s) for s in part.sub_parts().values())
         return all(safe(b) for b in self.blocks) and safe(self.final_norm) and safe(self.embedding) and safe(self.head_part)
+
 
     def cache_groups(self) -> List[CacheGroupSpec]:
         return [CacheGroupSpec(need, n) for need, n in zip(self.group_needs, self.group_layers)]
@@ -185,6 +214,10 @@ class DecoderModel:
             raise RuntimeError("the model has no weights yet")
         stream = ResidualStream(self.embedding.forward(step.token_ids, step))
         for entry, slot in zip(self.spec.run, slots):
+            if entry.add_vector is not None:
+                if stream.row_addend is not None:
+                    raise RuntimeError("a block left a pass vector unadded: its first norm must fold the stream")
+                stream.row_addend = self.pass_vectors.weight[entry.add_vector]   # the layer's first norm adds it
             stream = self.blocks[entry.layer].forward(stream, step, slot)
         if step.logit_rows.shape[0] == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)

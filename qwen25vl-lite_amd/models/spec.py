@@ -27,10 +27,15 @@ class LayerSpec:
 @dataclass(frozen=True)
 class RunEntry:
     """One step of the run list: run ``layer``.  ``cache_from`` names an earlier entry of the
-    run list whose cache this entry reads instead of writing its own."""
+    run list whose cache this entry reads instead of writing its own.  A layer that is named by
+    several entries runs with the same weights each time; every entry has a cache layer and a
+    state of its own unless it says ``cache_from``."""
 
     layer: int
     cache_from: Optional[int] = None
+    # a row of the model's pass vectors that is added to every token's residual sum right before
+    # this entry's layer runs
+    add_vector: Optional[int] = None
 
 
 @dataclass
@@ -54,3 +59,7 @@ class ModelSpec:
     # Their tensors go by ``embed_name`` / ``head_name`` with the last component replaced by the part's own names.
     embed: Optional[PartSpec] = None
     head: Optional[PartSpec] = None
+    # vectors that run entries add to the residual sum (``RunEntry.add_vector``): the canonical name
+    # of a tensor ``[rows, hidden]`` and its number of rows; None: the model has none
+    pass_vectors_name: Optional[str] = None
+    pass_vectors_rows: int = 0

@@ -13,7 +13,7 @@ import torch
 
 from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
 
-__all__ = ["residual_add", "gated_act", "softcap_", "group_norm_gate", "head_gate_", "qk_norm_rope_write"]
+__all__ = ["residual_add", "gated_act", "softcap_", "group_norm_gate", "head_gate_", "qk_norm_rope_write", "sandwich_norm"]
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 GATE_ACTS = {None: 0, "sigmoid": 1, "silu": 2}
@@ -104,23 +104,32 @@ def head_gate_(o: torch.Tensor, gate: torch.Tensor, num_heads: int) -> torch.Ten
 def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
                        cs: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                        v_cache: Optional[torch.Tensor], num_q_heads: int, num_kv_heads: int, head_dim: int,
-                       page_size: int, out_dtype: torch.dtype, *, interleaved: bool, values_are_keys: bool) -> torch.Tensor:
-    """Per head: RMS norm over the head (weights ``q_norm`` / ``k_norm`` of ``[head_dim]``, None: no
-    norm), then rotation by the angles whose ``(cos, sin)`` are ``cs [N, rot/2, 2]``: pairs
-    ``(2f, 2f+1)`` if ``interleaved``, else ``(f, f + rot/2)``.  Rotated queries are returned; rotated
-    keys and the values go into the page slots (``slots`` None: queries only).  ``x`` is float32
-    ``[N, >= (nq + nkv (+ nkv)) hd]``: query heads, key heads, and value heads unless
-    ``values_are_keys``, in which case a key head as projected (before norm and rotation) is its own value."""
-    _dev(x, q_norm, k_norm, cs, slots, k_cache, v_cache)
+                       page_size: int, out_dtype: torch.dtype, *, interleaved: bool, values_are_keys: bool,
+                       norm: Optional[str] = "before", bias: Optional[torch.Tensor] = None,
+                       value_dim: Optional[int] = None) -> torch.Tensor:
+    """Per head: ``bias`` (float32 over all columns, or None) is added; RMS norm over the head
+    (``norm`` ``"before"`` or ``"after"`` the rotation, None: no norm; weights ``q_norm`` / ``k_norm``
+    of ``[head_dim]``, None: a gain of one); rotation by the angles whose ``(cos, sin)`` are
+    ``cs [N, rot/2, 2]``: pairs ``(2f, 2f+1)`` if ``interleaved``, else ``(f, f + rot/2)``.  Rotated
+    queries are returned; rotated keys and the values go into the page slots (``slots`` None:
+    queries only).  ``x`` is float32 ``[N, >= nq hd + nkv hd (+ nkv vd)]``: query heads, key heads, and value
+    heads of ``value_dim`` channels unless ``values_are_keys``, in which case a key head as projected
+    (before norm and rotation) is its own value."""
+    _dev(x, q_norm, k_norm, cs, slots, k_cache, v_cache, bias)
     nq, nkv, hd = int(num_q_heads), int(num_kv_heads), int(head_dim)
+    vd = hd if value_dim is None else int(value_dim)
     write = slots is not None
     n = x.shape[0]
-    cols = (nq + (nkv * (1 if values_are_keys else 2) if write else 0)) * hd
+    cols = nq * hd + ((nkv * hd + (0 if values_are_keys else nkv * vd)) if write else 0)
     _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] >= cols and x.stride(1) == 1,
           "x must be float32 [N, at least the heads' columns]")
+    _need(norm in (None, "before", "after"), "the norm stands before or after the rotation, or is None")
+    _need(not (values_are_keys and vd != hd), "keys that are their own values have the keys' width")
     for w in (q_norm, k_norm):
         _need(w is None or (w.dtype == torch.float32 and w.shape == (hd,) and w.is_contiguous()),
               "a head norm's weight must be float32 [head_dim]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.dim() == 1 and bias.shape[0] >= cols
+                           and bias.is_contiguous()), "the bias must be float32 over the heads' columns")
     _need(cs.dtype == torch.float32 and cs.dim() == 3 and cs.is_contiguous() and cs.shape[0] >= n
           and cs.shape[2] == 2 and 2 * cs.shape[1] <= hd, "cs must be float32 [N, rot/2, 2] with rot <= head_dim")
     if write:
@@ -129,14 +138,50 @@ def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: 
               "the cache must have the activation dtype")
         _need(k_cache.is_contiguous() and k_cache.dim() == 4 and tuple(k_cache.shape[1:]) == (nkv, page_size, hd),
               "k_cache must be [pages, nkv, page_size, hd]")
-        _need(v_cache.is_contiguous() and tuple(v_cache.shape) == (k_cache.shape[0], nkv, hd, page_size),
-              "v_cache must be [pages, nkv, hd, page_size]")
+        _need(v_cache.is_contiguous() and tuple(v_cache.shape) == (k_cache.shape[0], nkv, vd, page_size),
+              "v_cache must be [pages, nkv, vd, page_size]")
     q_out = torch.empty((n, nq * hd), dtype=out_dtype, device=x.device)
     fn = _fn("gated", "qvl_qk_norm_rope_write",
-             [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
-              _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(x), x.stride(0), _ptr(q_norm), _ptr(k_norm), _ptr(cs), _ptr(slots), _ptr(q_out),
-              _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, n, nq, nkv, hd, cs.shape[1],
-              int(page_size), float(eps), int(interleaved), int(values_are_keys), int(write), dtype_code(out_dtype),
-              _stream()), "qk_norm_rope_write")
+             [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+              _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), x.stride(0), _ptr(bias), _ptr(q_norm), _ptr(k_norm), _ptr(cs), _ptr(slots), _ptr(q_out),
+              _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, n, nq, nkv, hd, vd, cs.shape[1],
+              int(page_size), float(eps), int(interleaved), int(values_are_keys), int(write),
+              {None: 0, "before": 1, "after": 2}[norm], dtype_code(out_dtype), _stream()), "qk_norm_rope_write")
     return q_out
+
+
+def sandwich_norm(h: torch.Tensor, y: Optional[torch.Tensor], gain: Optional[torch.Tensor], eps_y: float, factor: float,
+                  vec: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+                  rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``h += factor * rmsnorm(y) * gain + vec`` in float32 (``gain`` None: ``y`` is added as it is;
+    ``y`` None: nothing of it; ``vec`` None or one float32 vector for every row; ``y`` may be float32
+    slabs ``[slabs, N, H]``, added in order), then, if ``weight`` is given, ``rmsnorm(h) * weight`` in
+    ``out_dtype`` is returned.  With ``rows`` only those rows are formed and ``h`` is not written."""
+    _dev(h, y, gain, vec, weight, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [N, H]")
+    n, width = h.shape
+    nslabs, stride = 1, 0
+    if y is not None and y.dim() == 3:
+        _need(y.dtype == torch.float32 and tuple(y.shape[1:]) == (n, width) and y.is_contiguous(),
+              "slabs of y must be contiguous float32 [slabs, N, H]")
+        nslabs, stride = y.shape[0], n * width
+    elif y is not None:
+        _need(y.shape == h.shape and y.is_contiguous() and y.dtype in (torch.float32, torch.bfloat16),
+              "y must match h's shape, float32 or bfloat16")
+    for v in (gain, vec, weight):
+        _need(v is None or (v.dtype == torch.float32 and v.shape == (width,) and v.is_contiguous()),
+              "gains and vectors must be float32 [H]")
+    m = n
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be int32 [M]")
+        _need(weight is not None, "rows are chosen for a norm's output")
+        m = rows.shape[0]
+    out = None if weight is None else torch.empty((m, width), dtype=out_dtype, device=h.device)
+    fn = _fn("gated", "qvl_sandwich_norm",
+             [_c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr,
+              _c_int, _c_ptr, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(h), _ptr(y), dtype_code(y.dtype) if y is not None else 0, nslabs, stride, _ptr(gain), float(eps_y),
+              float(factor), _ptr(vec), _ptr(weight), float(eps), _ptr(out), dtype_code(out_dtype), _ptr(rows), m,
+              width, _stream()), "sandwich_norm")
+    return out

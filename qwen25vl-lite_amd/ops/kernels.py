@@ -201,9 +201,10 @@ def rope_kv_write(x: torch.Tensor, bias: Optional[torch.Tensor], positions: torc
     return q_out
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, freq_row: torch.Tensor, n: int) -> torch.Tensor:
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, freq_row: torch.Tensor, n: int,
+               amplitude: float = 1.0) -> torch.Tensor:
     """Cosine and sine of every token's rotation angle: float32 ``[n, rot/2, 2]`` with
-    ``(cos, sin)(positions[freq_row[f], i] * inv_freq[f])``, or ``(1, 0)`` where ``freq_row[f] < 0``."""
+    ``amplitude * (cos, sin)(positions[freq_row[f], i] * inv_freq[f])``, or ``(1, 0)`` where ``freq_row[f] < 0``."""
     _dev(positions, inv_freq, freq_row)
     rot_half = inv_freq.shape[0]
     _need(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "inv_freq must be float32 [rot/2]")
@@ -212,9 +213,9 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, freq_row: torch.
     _need(positions.dtype == torch.int32 and positions.dim() == 2 and positions.shape[1] >= n
           and positions.stride(1) == 1, "positions must be int32 [rows, N]")
     out = torch.empty((n, rot_half, 2), dtype=torch.float32, device=positions.device)
-    fn = _fn("elementwise", "qvl_rope_table", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+    fn = _fn("elementwise", "qvl_rope_table", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_ptr])
     _check(fn(_ptr(positions), positions.stride(0), _ptr(inv_freq), _ptr(freq_row), _ptr(out), int(n), rot_half,
-              _stream()), "rope_table")
+              float(amplitude), _stream()), "rope_table")
     return out
 
 
@@ -240,18 +241,22 @@ def copy_pages(cache: torch.Tensor, src: Sequence[int], dst: Sequence[int]) -> N
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             block_table: torch.Tensor, token_req: torch.Tensor, token_seqpos: torch.Tensor,
                             num_q_heads: int, window: Optional[int], scale: float,
-                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            out: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
     """Attention of every token over its request's pages; any head size, float32 arithmetic.
 
     ``q`` is ``[N, nq hd]``; token ``n`` belongs to row ``token_req[n]`` of ``block_table`` and
-    sits at sequence index ``token_seqpos[n]``; it sees keys ``max(0, p - window + 1) .. p``.
+    sits at sequence index ``token_seqpos[n]``; it sees keys ``max(0, p - window + 1) .. p`` and,
+    with a window, the first ``keep_first`` keys of its request.  The result is ``[N, nq vd]``,
+    ``vd`` being the value width of ``v_cache [pages, nkv, vd, page_size]``.
     """
     _dev(q, k_cache, v_cache, block_table, token_req, token_seqpos, out)
     n = q.shape[0]
     nq = int(num_q_heads)
     _need(k_cache.dim() == 4 and k_cache.is_contiguous() and v_cache.is_contiguous(), "cache must be contiguous")
     pages, nkv, ps, hd = k_cache.shape
-    _need(tuple(v_cache.shape) == (pages, nkv, hd, ps), "v_cache must be [pages, nkv, hd, page_size]")
+    _need(v_cache.dim() == 4 and tuple(v_cache.shape[:2]) == (pages, nkv) and v_cache.shape[3] == ps,
+          "v_cache must be [pages, nkv, vd, page_size]")
+    vd = v_cache.shape[2]
     _need(q.shape == (n, nq * hd) and q.is_contiguous() and q.dtype == k_cache.dtype == v_cache.dtype,
           "q must be [N, nq hd] in the cache's dtype")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
@@ -259,14 +264,16 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     for t in (token_req, token_seqpos):
         _need(t.dtype == torch.int32 and t.shape == (n,) and t.is_contiguous(), "token maps must be int32 [N]")
     if out is None:
-        out = torch.empty_like(q)
-    _need(out.shape == q.shape and out.dtype == q.dtype and out.is_contiguous(), "out must match q")
+        out = torch.empty((n, nq * vd), dtype=q.dtype, device=q.device)
+    _need(out.shape == (n, nq * vd) and out.dtype == q.dtype and out.is_contiguous(), "out must be [N, nq vd]")
+    _need(keep_first >= 0, "keep_first cannot be negative")
     fn = _fn("attention_generic", "qvl_attn_generic",
              [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
-              _c_int, _c_int, _c_float, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr])
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(token_req),
-              _ptr(token_seqpos), _ptr(out), n, nq, nkv, hd, ps, int(window or 0), float(scale),
-              dtype_code(q.dtype), _stream()), "paged_attention_generic")
+              _ptr(token_seqpos), _ptr(out), n, nq, nkv, hd, vd, ps, int(window or 0),
+              int(keep_first) if window else 0, float(scale), dtype_code(q.dtype), _stream()),
+           "paged_attention_generic")
     return out
 
 

@@ -37,8 +37,14 @@ class PagedAttention(Mixer):
     rotation, is its own value), ``head_gate`` (each head's output is multiplied by the sigmoid of
     one number per head, a projection ``g`` of ``[heads, hidden]`` of the mixer's input), ``names``
     (local names of the tensors' owners, default ``q_proj`` ... ``o_proj``, ``g_proj``, ``q_norm``,
-    ``k_norm``).  A position encoding may ask for interleaved pairs (``interleaved``).  Any of these
-    takes the projection through float32 and one kernel that norms, rotates and writes the cache."""
+    ``k_norm``, ``v``).  A position encoding may ask for interleaved pairs (``interleaved``).
+    ``qk_norm_where`` (``"before"``, the default, or ``"after"`` the rotation) and ``qk_norm_weights``
+    (False: the norm has no gains and the mixer no such tensors), ``value_dim`` (values of another
+    width than keys), ``keep_first`` (with a window: the first so many keys of a request stay visible
+    to every later token, at their true positions), ``element_gate`` (the concatenated heads are
+    multiplied element by element by the sigmoid of a projection ``g`` of ``[heads value_dim, hidden]``),
+    ``out_bias`` (the output projection has a bias).  Any of these except the last takes the
+    projection through float32 and one kernel that norms, rotates and writes the cache."""
 
     graph_safe = True
     takes_lazy_norm = True
@@ -56,8 +62,22 @@ class PagedAttention(Mixer):
         self.kv_shared = bool(params.get("kv_shared", False))
         eps = params.get("qk_norm_eps")
         self.qk_norm_eps: Optional[float] = None if eps is None else float(eps)
+        self.qk_norm_where = str(params.get("qk_norm_where", "before"))
+        self.qk_norm_weights = bool(params.get("qk_norm_weights", True))
         self.values_are_keys = bool(params.get("values_are_keys", False))
         self.head_gate = bool(params.get("head_gate", False))
+        self.element_gate = bool(params.get("element_gate", False))
+        self.out_bias = bool(params.get("out_bias", False))
+        self.vd = int(params.get("value_dim") or self.hd)
+        self.keep_first = int(params.get("keep_first") or 0) if self.window else 0
+        if self.qk_norm_where not in ("before", "after"):
+            raise ValueError("qk_norm_where is 'before' or 'after' (the rotation)")
+        if self.head_gate and self.element_gate:
+            raise ValueError("an attention mixer has one kind of output gate at most")
+        if self.values_are_keys and self.vd != self.hd:
+            raise ValueError("keys that are their own values have the keys' width")
+        if self.keep_first < 0:
+            raise ValueError("keep_first cannot be negative")
         names = dict(params.get("names") or {})
         self.names = {k: names.get(k, d) for k, d in (("q", "q_proj"), ("k", "k_proj"), ("v", "v_proj"), ("o", "o_proj"),
                                                       ("g", "g_proj"), ("q_norm", "q_norm"), ("k_norm", "k_norm"))}
@@ -69,13 +89,15 @@ class PagedAttention(Mixer):
         self.position = build_part("position", pos, dtype, device)
         self.interleaved = bool(getattr(self.position, "interleaved", False))
         self.normed_path = (self.qk_norm_eps is not None or self.values_are_keys or self.head_gate
-                            or self.interleaved)
+                            or self.element_gate or self.interleaved or self.vd != self.hd)
+        self.gate_rows = self.nq if self.head_gate else (self.nq * self.vd if self.element_gate else 0)
         self.w_in: Optional[torch.Tensor] = None
         self.b_in: Optional[torch.Tensor] = None
         self.w_out: Optional[torch.Tensor] = None
+        self.b_out: Optional[torch.Tensor] = None
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.nkv, self.hd, self.window)
+        return CacheNeed(self.nkv, self.hd, self.window, self.keep_first, None if self.vd == self.hd else self.vd)
 
     def _projections(self):
         """``(role, rows)`` of the matrices stacked into the input product, in order."""
@@ -83,7 +105,7 @@ class PagedAttention(Mixer):
         if not self.kv_shared:
             out.append(("k", self.nkv * self.hd))
             if not self.values_are_keys:
-                out.append(("v", self.nkv * self.hd))
+                out.append(("v", self.nkv * self.vd))
         return out
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -94,13 +116,15 @@ class PagedAttention(Mixer):
         if self.qkv_bias:
             for role, rows in self._projections():
                 specs[f"{n[role]}.bias"] = ParamSpec((rows,), "vector")
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             specs[f"{n['q_norm']}.weight"] = ParamSpec((self.hd,), "vector", init="around_one")
             if not self.kv_shared:
                 specs[f"{n['k_norm']}.weight"] = ParamSpec((self.hd,), "vector", init="around_one")
-        if self.head_gate:
-            specs[f"{n['g']}.weight"] = ParamSpec((self.nq, self.hidden))
-        specs[f"{n['o']}.weight"] = ParamSpec((self.hidden, self.nq * self.hd))
+        if self.gate_rows:
+            specs[f"{n['g']}.weight"] = ParamSpec((self.gate_rows, self.hidden))
+        specs[f"{n['o']}.weight"] = ParamSpec((self.hidden, self.nq * self.vd))
+        if self.out_bias:
+            specs[f"{n['o']}.bias"] = ParamSpec((self.hidden,), "vector")
         return specs
 
     def load(self, tensors):
@@ -109,14 +133,15 @@ class PagedAttention(Mixer):
         # One product for q, k and v (and the heads' gate): the matrices are stacked by rows.
         mats = [tensors[f"{n[r]}.weight"] for r in roles]
         bias = [tensors[f"{n[r]}.bias"] for r in roles] if self.qkv_bias else None
-        if self.head_gate:
+        if self.gate_rows:
             mats.append(tensors[f"{n['g']}.weight"])
             if bias is not None:
-                bias.append(torch.zeros(self.nq, dtype=bias[0].dtype, device=bias[0].device))
+                bias.append(torch.zeros(self.gate_rows, dtype=bias[0].dtype, device=bias[0].device))
         self.w_in = torch.cat(mats, dim=0).contiguous()
         self.b_in = torch.cat(bias).contiguous() if bias is not None else None
         self.w_out = tensors[f"{n['o']}.weight"]
-        if self.qk_norm_eps is not None:
+        self.b_out = tensors.get(f"{n['o']}.bias")
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             self.q_norm = tensors[f"{n['q_norm']}.weight"]
             self.k_norm = tensors.get(f"{n['k_norm']}.weight")
 
@@ -129,8 +154,10 @@ class PagedAttention(Mixer):
             if self.b_in is not None:
                 out[f"{n[role]}.bias"] = self.b_in[row:row + rows]
             row += rows
-        if self.head_gate:
-            out[f"{n['g']}.weight"] = self.w_in[row:row + self.nq]
+        if self.gate_rows:
+            out[f"{n['g']}.weight"] = self.w_in[row:row + self.gate_rows]
+        if self.b_out is not None:
+            out[f"{n['o']}.bias"] = self.b_out
         if self.q_norm is not None:
             out[f"{n['q_norm']}.weight"] = self.q_norm
         if self.k_norm is not None:
@@ -152,8 +179,16 @@ class PagedAttention(Mixer):
         q = self._project_few_rows(x, step, group, slot, write, inv_freq, freq_row)
         if q is None:
             q = self._project(x, step, group, slot, write, inv_freq, freq_row)
-        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
-        return linear_into(step.residual, o, self.w_out)
+        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale,
+                            keep_first=self.keep_first)
+        return self._output(o, step)
+
+    def _output(self, o: torch.Tensor, step: StepContext):
+        """The output projection: into the residual where the block offers it and there is no bias."""
+        if self.b_out is None:
+            return linear_into(step.residual, o, self.w_out)
+        return linear(o, self.w_out, self.b_out,
+                      out_dtype=torch.float32 if o.shape[0] <= skinny.ONE_BLOCK_ROWS else None)
 
     def _forward_normed(self, x, step, group, slot, write, inv_freq, freq_row):
         """The path with a per-head norm, interleaved pairs, keys as values or a gate per head: the
@@ -161,18 +196,21 @@ class PagedAttention(Mixer):
         keys and writes keys and values into the pages, and the gate multiplies the heads' outputs."""
         from ..ops import gated
 
-        proj = linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
+        proj = linear(x, self.w_in, out_dtype=torch.float32)     # the bias is added by the kernel that norms
         cs = self._rotation_table(step, inv_freq, freq_row, proj.shape[0])
         q = gated.qk_norm_rope_write(
             proj, self.q_norm, self.k_norm, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0, cs,
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
             self.nq, self.nkv, self.hd, group.page_size, self.dtype, interleaved=self.interleaved,
-            values_are_keys=self.values_are_keys)
-        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale)
-        if self.head_gate:
-            at = self.w_in.shape[0] - self.nq
-            gated.head_gate_(o, proj[:, at:at + self.nq], self.nq)
-        return linear_into(step.residual, o, self.w_out)
+            values_are_keys=self.values_are_keys, norm=None if self.qk_norm_eps is None else self.qk_norm_where,
+            bias=self.b_in, value_dim=self.vd)
+        o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale,
+                            keep_first=self.keep_first)
+        if self.gate_rows:
+            # one gate per head, or one per element (a "head" of one channel)
+            at = self.w_in.shape[0] - self.gate_rows
+            gated.head_gate_(o, proj[:, at:at + self.gate_rows], self.gate_rows)
+        return self._output(o, step)
 
     def _project(self, x, step, group, slot, write, inv_freq, freq_row) -> torch.Tensor:
         # Projections are written out in float32 (the accumulator, unrounded): bias, rotation and
@@ -197,7 +235,8 @@ class PagedAttention(Mixer):
         key = ("rope_cs", self.position.table_key(self.hd))
         cs = step.per_pass.get(key)
         if cs is None:
-            cs = step.per_pass[key] = kernels.rope_table(step.positions, inv_freq, freq_row, n)
+            cs = step.per_pass[key] = kernels.rope_table(step.positions, inv_freq, freq_row, n,
+                                                         amplitude=float(getattr(self.position, "amplitude", 1.0)))
         return cs
 
     def _project_few_rows(self, x, step, group, slot, write, inv_freq, freq_row) -> Optional[torch.Tensor]:

@@ -61,11 +61,19 @@ class PartSpec:
 @dataclass(frozen=True)
 class CacheNeed:
     """Keys and values a mixer keeps per token.  ``window`` None: all keys stay; a number:
-    only the last ``window`` keys are read, older pages may be given back."""
+    only the last ``window`` keys are read, older pages may be given back, except the pages of
+    the first ``keep_first`` tokens, which every later token still reads.  ``value_dim`` None:
+    values are as wide as keys (``head_dim``)."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    keep_first: int = 0
+    value_dim: Optional[int] = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -83,7 +91,7 @@ class LayerSlot:
 
     group: Optional[int] = None
     k_cache: Optional[torch.Tensor] = None  # [pages, nkv, page_size, hd]
-    v_cache: Optional[torch.Tensor] = None  # [pages, nkv, hd, page_size]
+    v_cache: Optional[torch.Tensor] = None  # [pages, nkv, vd, page_size]
     writes: bool = True
     state: Optional[torch.Tensor] = None    # [max_num_seqs, *StateNeed.shape]
     # a block with several mixers: each one's slot under the mixer's sub-part name (this slot is
@@ -136,6 +144,11 @@ class ResidualStream:
 
     h: torch.Tensor                          # float32 [N, hidden]
     pending: Optional[torch.Tensor] = None   # float32 or run dtype [N, hidden]
+    # (gain float32 [hidden], eps, factor): the pending addend enters the sum as
+    # factor * rmsnorm(pending) * gain instead of as it is (a sublayer with a norm behind it)
+    pending_norm: Optional[Tuple[torch.Tensor, float, float]] = None
+    # a vector float32 [hidden] that the next norm adds to every row of the sum
+    row_addend: Optional[torch.Tensor] = None
 
 
 class Part:

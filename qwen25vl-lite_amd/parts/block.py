@@ -6,7 +6,7 @@ from typing import Dict, Optional
 
 from .base import Block, LayerSlot, Part, PartSpec, ResidualStream, StepContext, build_part, register_part
 
-__all__ = ["PreNormBlock", "ParallelBlock"]
+__all__ = ["PreNormBlock", "ParallelBlock", "SandwichBlock"]
 
 
 class PreNormBlock(Block):
@@ -84,5 +84,55 @@ class ParallelBlock(Block):
         return stream
 
 
+class SandwichBlock(Block):
+    """``h += m * norm1b(mixer(norm1(h))); h += m * norm2b(ffn(norm2(h)))``: a norm before and one
+    behind each sublayer, and a fixed factor ``m`` on what joins the sum.
+
+    params: ``norm1``, ``mixer``, ``norm1b``, ``norm2``, ``ffn``, ``norm2b`` (:class:`PartSpec` each; ``ffn``
+    None for a layer without a feed-forward, whose ``norm2`` and ``norm2b`` are then not built),
+    ``residual_mult`` (``m``, default 1) and ``names``, the checkpoint sub-name of each part.  The
+    norms behind the sublayers are RMS norms: a sublayer's result waits in the stream with that
+    norm's gain, and the kernel of the next norm in line forms the normed addend, the float32 sum
+    and its own output in one pass.
+    """
+
+    graph_safe = True
+
+    def __init__(self, params, dtype, device):
+        super().__init__(dtype, device)
+        self.names: Dict[str, str] = dict(params["names"])
+        self.mult = float(params.get("residual_mult", 1.0))
+        self.norm1 = build_part("norm", params["norm1"], dtype, device)
+        self.mixer = build_part("mixer", params["mixer"], dtype, device)
+        self.norm1b = build_part("norm", params["norm1b"], dtype, device)
+        self.ffn: Optional[Part] = None
+        if params.get("ffn") is not None:
+            self.norm2 = build_part("norm", params["norm2"], dtype, device)
+            self.ffn = build_part("ffn", params["ffn"], dtype, device)
+            self.norm2b = build_part("norm", params["norm2b"], dtype, device)
+        for post in (self.norm1b, getattr(self, "norm2b", None)):
+            if post is not None and not (hasattr(post, "weight") and hasattr(post, "eps")):
+                raise ValueError("the norm behind a sublayer must be an RMS norm")
+
+    def sub_parts(self) -> Dict[str, Part]:
+        parts = {self.names["norm1"]: self.norm1, self.names["mixer"]: self.mixer, self.names["norm1b"]: self.norm1b}
+        if self.ffn is not None:
+            parts.update({self.names["norm2"]: self.norm2, self.names["ffn"]: self.ffn,
+                          self.names["norm2b"]: self.norm2b})
+        return parts
+
+    def forward(self, stream: ResidualStream, step: StepContext, slot: LayerSlot) -> ResidualStream:
+        x = self.norm1.forward(stream)
+        step.residual = None                 # a sublayer's result is normed before it joins the sum
+        stream.pending = self.mixer.forward(x, step, slot)
+        stream.pending_norm = (self.norm1b.weight, self.norm1b.eps, self.mult)
+        if self.ffn is not None:
+            y = self.norm2.forward(stream)
+            stream.pending = self.ffn.forward(y, step)
+            stream.pending_norm = (self.norm2b.weight, self.norm2b.eps, self.mult)
+        return stream
+
+
+register_part("block", "sandwich", SandwichBlock)
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "parallel", ParallelBlock)

@@ -38,6 +38,16 @@ class RMSNorm(Norm):
         self.weight = stored + self.offset if self.offset else stored
 
     def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
+        if stream.pending_norm is not None or stream.row_addend is not None:
+            # an addend that is normed on its way into the sum, or a vector for every row: one kernel
+            # forms the sum and this norm
+            from ..ops.gated import sandwich_norm
+            gain, eps_y, factor = stream.pending_norm or (None, 0.0, 1.0)
+            out = sandwich_norm(stream.h, stream.pending, gain if stream.pending is not None else None, eps_y, factor,
+                                stream.row_addend, self.weight, self.eps, self.dtype, rows=rows)
+            if rows is None:
+                stream.pending = stream.pending_norm = stream.row_addend = None
+            return out
         if (lazy and rows is None and stream.pending is None and self.dtype == torch.bfloat16
                 and self.size % 8 == 0 and skinny.folds_norm(stream.h.shape[0], self.size, stream.h.device)):
             # a decode step: the product that follows computes the norm on the way

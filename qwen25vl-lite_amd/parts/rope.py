@@ -20,7 +20,7 @@ import torch
 
 from .base import PositionEncoding, register_part
 
-__all__ = ["MRoPE", "RoPE1D", "inverse_frequencies", "rescale_frequencies"]
+__all__ = ["MRoPE", "RoPE1D", "inverse_frequencies", "rescale_frequencies", "ramp_frequencies"]
 
 
 def inverse_frequencies(rotary_dim: int, theta: float) -> torch.Tensor:
@@ -75,9 +75,30 @@ def rescale_frequencies(freqs: torch.Tensor, factor: float, low: float, high: fl
     return torch.where(wavelength < original / high, f, torch.where(wavelength > original / low, f / factor, blended))
 
 
+def ramp_frequencies(freqs: torch.Tensor, theta: float, factor: float, original: int, fast: float, slow: float):
+    """Frequencies stretched by a ramp over the channel index, and the factor that goes on every
+    cosine and sine.  With ``d = 2 len(freqs)`` rotated channels, a frequency that makes ``t`` turns
+    over the ``original`` length sits at index ``i(t) = d ln(original / (2 pi t)) / (2 ln theta)``;
+    ``lo = max(floor(i(fast)), 0)``, ``hi = min(ceil(i(slow)), d - 1)``, ``r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``;
+    frequency ``i`` becomes ``f_i / factor * r_i + f_i (1 - r_i)`` and the amplitude is
+    ``0.1 ln(factor) + 1``.  Computed in float64."""
+    f = freqs.to(torch.float64)
+    d = 2 * f.shape[0]
+
+    def index_of(turns: float) -> float:
+        return d * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+
+    lo = max(math.floor(index_of(fast)), 0)
+    hi = min(math.ceil(index_of(slow)), d - 1)
+    ramp = ((torch.arange(f.shape[0], dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp), 0.1 * math.log(factor) + 1.0
+
+
 class RoPE1D(PositionEncoding):
     """params: ``theta``, optional ``rotary_dim`` (default: the whole head), optional ``scaling``
-    (``factor``, ``low``, ``high``, ``original``: see :func:`rescale_frequencies`), optional
+    (``factor``, ``low``, ``high``, ``original``: see :func:`rescale_frequencies`; or ``kind: "ramp"``
+    with ``factor``, ``original``, ``fast``, ``slow``: see :func:`ramp_frequencies`, which also scales
+    the cosines and sines: ``amplitude``), optional
     ``interleaved`` (True: channel 2f is rotated with channel 2f+1; default: f with f + rot/2.  The
     kernel that rotates reads it from the encoding)."""
 
@@ -91,21 +112,32 @@ class RoPE1D(PositionEncoding):
         self.rotary_dim = params.get("rotary_dim")
         self.interleaved = bool(params.get("interleaved", False))
         sc = params.get("scaling")
-        self.scaling = None if not sc else (float(sc["factor"]), float(sc["low"]), float(sc["high"]),
-                                            int(sc["original"]))
-        if self.scaling is not None and not (self.scaling[0] > 0 and self.scaling[2] > self.scaling[1]):
-            raise ValueError("frequency scaling needs a positive factor and high > low")
+        self.scaling = None
+        self.ramp = None
+        self.amplitude = 1.0
+        if sc and sc.get("kind") == "ramp":
+            self.ramp = (float(sc["factor"]), int(sc["original"]), float(sc["fast"]), float(sc["slow"]))
+            if not (self.ramp[0] > 0 and self.ramp[2] > 0 and self.ramp[3] > 0 and self.theta > 1):
+                raise ValueError("a frequency ramp needs a positive factor and turn counts, and a base above 1")
+            self.amplitude = 0.1 * math.log(self.ramp[0]) + 1.0
+        elif sc:
+            self.scaling = (float(sc["factor"]), float(sc["low"]), float(sc["high"]), int(sc["original"]))
+            if not (self.scaling[0] > 0 and self.scaling[2] > self.scaling[1]):
+                raise ValueError("frequency scaling needs a positive factor and high > low")
         self._tables = {}
 
     def table_key(self, head_dim: int):
-        return ("rope", self.theta, self.rotary_dim, self.scaling, head_dim)
+        return ("rope", self.theta, self.rotary_dim, self.scaling, self.ramp, head_dim)
 
     def rotary_tables(self, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
         if head_dim not in self._tables:
             rot = int(self.rotary_dim) if self.rotary_dim is not None else head_dim
             if rot % 2 or rot > head_dim:
                 raise ValueError(f"rotary_dim {rot} must be even and at most the head size {head_dim}")
-            if self.scaling is None:
+            if self.ramp is not None:
+                idx = torch.arange(0, rot, 2, dtype=torch.float64)
+                freqs = ramp_frequencies(float(self.theta) ** (-idx / rot), self.theta, *self.ramp)[0].to(torch.float32)
+            elif self.scaling is None:
                 freqs = inverse_frequencies(rot, self.theta)
             else:
                 idx = torch.arange(0, rot, 2, dtype=torch.float64)
