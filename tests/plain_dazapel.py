@@ -149,9 +149,31 @@ def route(z: torch.Tensor, top: int, groups: int, keep: int, scale: float):
     return chosen, w / (w.sum(-1, keepdim=True) + WEIGHT_FLOOR) * scale
 
 
-def moe(h: torch.Tensor, t: Dict[str, torch.Tensor], p: str, mlp: dict, store: Callable = _keep) -> torch.Tensor:
+def choice_margin(z: torch.Tensor, top: int, groups: int, keep: int) -> torch.Tensor:
+    """Per token, by how much the router's choice is clear: the gap between the last group kept and
+    the first one left out, and between the last expert chosen and the best allowed one left out
+    (infinite where nothing is left out)."""
+    T, E = z.shape
+    s = torch.sigmoid(z)
+    per = E // groups
+    gscore = s.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1).sort(dim=-1, descending=True)
+    margin = torch.full((T,), float("inf"), dtype=z.dtype)
+    if keep < groups:
+        margin = gscore.values[:, keep - 1] - gscore.values[:, keep]
+    allowed = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, gscore.indices[:, :keep], True)
+    masked = torch.where(allowed[:, :, None].expand(T, groups, per).reshape(T, E), s, torch.full_like(s, -1.0))
+    if top < keep * per:
+        ranked = masked.sort(dim=-1, descending=True).values
+        margin = torch.minimum(margin, ranked[:, top - 1] - ranked[:, top])
+    return margin
+
+
+def moe(h: torch.Tensor, t: Dict[str, torch.Tensor], p: str, mlp: dict, store: Callable = _keep,
+        margins: Optional[list] = None) -> torch.Tensor:
     r = mlp["router"]
     z = h @ t[p + "router"].T
+    if margins is not None:
+        margins.append(choice_margin(z, int(r["top"]), int(r["groups"]["count"]), int(r["groups"]["keep"])))
     chosen, w = route(z, int(r["top"]), int(r["groups"]["count"]), int(r["groups"]["keep"]), float(r["scale"]))
     out = torch.zeros(h.shape[0], t[p + "e0.down"].shape[0], dtype=h.dtype)
     limit = float(mlp["expert"]["limit"])
@@ -184,8 +206,9 @@ def run_order(cfg: dict) -> List[tuple]:
 
 
 def dazapel_forward(cfg: dict, t: Dict[str, torch.Tensor], tokens, store: Callable = _keep,
-                    trace: Optional[list] = None) -> torch.Tensor:
-    """Logits ``[T, vocab]`` of a whole sequence.  ``trace`` collects the residual after every layer run."""
+                    trace: Optional[list] = None, margins: Optional[list] = None) -> torch.Tensor:
+    """Logits ``[T, vocab]`` of a whole sequence.  ``trace`` collects the residual after every layer
+    run, ``margins`` every router's :func:`choice_margin` per token."""
     eps, mult = float(cfg["norm"]["eps"]), float(cfg["residual_mult"])
     x = t["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     for i, pass_no in run_order(cfg):
@@ -197,7 +220,7 @@ def dazapel_forward(cfg: dict, t: Dict[str, torch.Tensor], tokens, store: Callab
         y = attention_mixer(store(rms_norm(x, t[p + "norm1"], eps)), t, p + "mix.", layer["mixer"], eps, store)
         x = x + mult * rms_norm(y, t[p + "norm1b"], eps)
         if layer.get("mlp") is not None:
-            y = moe(store(rms_norm(x, t[p + "norm2"], eps)), t, p + "mlp.", layer["mlp"], store)
+            y = moe(store(rms_norm(x, t[p + "norm2"], eps)), t, p + "mlp.", layer["mlp"], store, margins)
             x = x + mult * rms_norm(y, t[p + "norm2b"], eps)
         if trace is not None:
             trace.append(x.clone())
