@@ -16,13 +16,20 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """Attention of the step's tokens over their requests' pages.
 
     bfloat16 with a head size in steps of 16 runs on the matrix cores; everything else
-    (float32, other head sizes, values of another width than the keys, a window that keeps the
-    first keys) runs through the float32-arithmetic kernel.
+    bfloat16 with a window that keeps the first keys, or values of another width than the keys, has a
+    matrix-core kernel of its own; everything else (float32, other head sizes) runs through the
+    float32-arithmetic kernel.
     """
     plain = not (window and keep_first) and v_cache.shape[2] == k_cache.shape[3]
     if q.dtype == torch.bfloat16 and plain:
         from . import attention_mfma
         out = attention_mfma.try_attention(q, k_cache, v_cache, block_table, step, num_q_heads, window, scale)
+        if out is not None:
+            return out
+    elif q.dtype == torch.bfloat16:
+        from . import attention_window
+        out = attention_window.try_attention(q, k_cache, v_cache, block_table, step, num_q_heads, window, keep_first,
+                                             scale)
         if out is not None:
             return out
     return kernels.paged_attention_generic(q, k_cache, v_cache, block_table, step.token_req, step.token_seqpos,

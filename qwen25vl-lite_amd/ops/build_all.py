@@ -35,6 +35,12 @@ LIBRARIES = [
     ("attention_mfma", {"HD": 64}),
     ("attention_mfma", {"HD": 96}),
     ("attention_mfma", {"HD": 112}),
+    # the matrix-core attention for windows that keep the first keys is compiled per key and value size
+    ("attention_window", {"HD": 128, "VD": 128}),
+    ("attention_window", {"HD": 16, "VD": 24}),
+    ("attention_window", {"HD": 48, "VD": 16}),
+    ("attention_window", {"HD": 16, "VD": 16}),
+    ("attention_window", {"HD": 64, "VD": 32}),
     # the kind whose waves carry three column tiles (long prompts)
     ("attention_mfma", {"HD": 128, "BLK_CT": 3}),
     ("attention_mfma", {"HD": 48, "BLK_CT": 3}),

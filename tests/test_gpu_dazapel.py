@@ -330,3 +330,62 @@ def test_bfloat16_generation_from_graphs_matches_eager_steps(folders):
             outs.append([o.output_token_ids for o in
                          llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))])
     assert outs[0] == outs[1]
+
+
+# ---------------------------------------------------------------------------------------------
+# the matrix-core attention for windows that keep the first keys
+# ---------------------------------------------------------------------------------------------
+def _paged_case(runs, hd, vd, nkv, ps, seed):
+    """Requests of (tokens already cached, tokens in this step): keys and values in shuffled pages."""
+    import types
+    g = torch.Generator().manual_seed(seed)
+    ctx = [a + b for a, b in runs]
+    need = [(c + ps - 1) // ps for c in ctx]
+    perm = torch.randperm(sum(need) + 3, generator=g).tolist()
+    width = max(need)
+    table = torch.full((len(runs), width), -1, dtype=torch.int32)
+    k_cache = torch.zeros(sum(need) + 3, nkv, ps, hd)
+    v_cache = torch.zeros(sum(need) + 3, nkv, vd, ps)
+    keys, values = [], []
+    for r, c in enumerate(ctx):
+        k, v = torch.randn(c, nkv, hd, generator=g), torch.randn(c, nkv, vd, generator=g)
+        keys.append(k.to(torch.bfloat16).float())
+        values.append(v.to(torch.bfloat16).float())
+        for i in range(need[r]):
+            page = perm.pop()
+            table[r, i] = page
+            n = min(ps, c - i * ps)
+            k_cache[page, :, :n] = keys[r][i * ps:i * ps + n].transpose(0, 1)
+            v_cache[page, :, :, :n] = values[r][i * ps:i * ps + n].permute(1, 2, 0)
+    cu = [0]
+    for _, b in runs:
+        cu.append(cu[-1] + b)
+    step = types.SimpleNamespace(
+        num_reqs=len(runs), cu_q=torch.tensor(cu, dtype=torch.int32).cuda(), ctx_len=torch.tensor(ctx, dtype=torch.int32).cuda(),
+        cu_q_host=cu, ctx_len_host=ctx, max_q_len=max(b for _, b in runs), max_ctx_len=max(ctx), derived={})
+    return step, table.cuda(), k_cache.to(torch.bfloat16).cuda(), v_cache.to(torch.bfloat16).cuda(), keys, values
+
+
+@pytest.mark.parametrize("hd, vd, nq, nkv, ps", [(16, 24, 4, 2, 16), (48, 16, 3, 1, 16), (128, 128, 8, 2, 16), (64, 32, 20, 1, 8),
+                                                 (16, 16, 2, 2, 48)])
+@pytest.mark.parametrize("window, keep", [(9, 3), (40, 20), (70, 0), (33, 100), (None, 0)])
+def test_window_attention_on_the_matrix_cores(hd, vd, nq, nkv, ps, window, keep):
+    """Prompt portions that start anywhere and decoded tokens, a wave per tile and four waves sharing a tile,
+    against dense masked attention: windows that end inside a block of keys, kept keys that reach into
+    the window, pages in shuffled order."""
+    from qwen25vl_lite_amd.ops.attention_window import try_attention
+    for runs in ([(0, 75), (130, 1), (37, 2), (95, 41), (0, 1)], [(199, 1), (64, 1), (3, 1)]):
+        step, table, kc, vc, keys, values = _paged_case(runs, hd, vd, nkv, ps, seed=hd + (window or 0))
+        n = step.cu_q_host[-1]
+        q = torch.randn(n, nq, hd, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+        scale = 2.0 * hd ** -0.5
+        want = torch.empty(n, nq, vd)
+        for r, (before, now) in enumerate(runs):
+            see = plain.visible(before + now, window, keep)[before:]
+            for h in range(nq):
+                s = (q[step.cu_q_host[r]:step.cu_q_host[r + 1], h].float() @ keys[r][:, h // (nq // nkv)].T) * scale
+                want[step.cu_q_host[r]:step.cu_q_host[r + 1], h] = torch.softmax(s.masked_fill(~see, float("-inf")), -1) @ values[r][:, h // (nq // nkv)]
+        for share in (False, True):
+            got = try_attention(q.reshape(n, nq * hd).cuda(), kc, vc, table, step, nq, window, keep, scale, share=share)
+            assert got is not None
+            assert torch.allclose(got.float().cpu().view(n, nq, vd), want, atol=2e-2, rtol=2e-2), (runs, share)
