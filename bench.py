@@ -71,6 +71,30 @@ def gogudra_config(layers, size="7b", order=("gla", "gla", "lightning", "attenti
                        for i in range(int(layers))]}
 
 
+def dazapel_config(layers, size="7b", experts=32, top=6, window=1024, keep_first=4):
+    """A Dazapel decoder with the width, head counts and vocabulary of one of SIZES and heads of 128
+    channels.  Every layer has routed experts of an eighth of the size's feed-forward width, of which a
+    token uses ``top``, and a shared expert twice as wide: with the default ``top`` of 6 a token runs
+    through as many feed-forward channels as in the dense decoder.  Odd layers see the last ``window``
+    keys and a request's first ``keep_first``; even layers see everything."""
+    s = SIZES[size]
+    nh, nkv, hd = s["num_attention_heads"], s["num_key_value_heads"], 128
+    ff = s["intermediate_size"] // 8 // 16 * 16
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": 2 * ff, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 8, "keep": 4}}}
+
+    def mixer(i):
+        m = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+             "rot": {"base": 500000.0, "dims": hd // 2,
+                     "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+        if i % 2:
+            m["mask"] = {"size": window, "keep_first": keep_first}
+        return m
+
+    return {"architecture": "Dazapel", "width": s["hidden_size"], "vocab": s["vocab_size"], "norm": {"eps": 1e-6},
+            "residual_mult": 0.5, "layers": [{"type": "attention", "mixer": mixer(i), "mlp": mlp} for i in range(int(layers))]}
+
+
 def step_bytes(t, batch, ctx, bytes_per_value=2):
     """Bytes a decode step has to read: every weight it uses once (all layers and the head; of the
     embedding only the rows looked up) and the keys and values of the live requests."""
@@ -225,7 +249,7 @@ def main(argv=None) -> int:
     ap.add_argument("--attention", type=int, nargs="+", metavar="TOKENS",
                     help="instead: the prefill attention alone (one request of that many tokens in one step, the "
                          "chosen size's heads, bfloat16, pages in shuffled order), microseconds and TFLOP/s for each length")
-    ap.add_argument("--design", choices=["gogudra"],
+    ap.add_argument("--design", choices=["gogudra", "dazapel"],
                     help="instead: prefill (2,048 tokens) and decode throughput of this design at the chosen size's "
                          "width, heads and feed-forward (random weights), beside the Qwen2.5-VL decoder with as many layers")
     ap.add_argument("--order", default="gla,gla,lightning,attention",
@@ -328,14 +352,15 @@ def main(argv=None) -> int:
         from qwen25vl_lite_amd.config import load_config
         out = {"metric": f"prefill and decode tok/s, {args.design} beside the Qwen2.5-VL decoder "
                          f"({args.size} sizes, {args.layers} layers, {args.dtype})", "unit": "tokens/s",
-               "order": args.order.split(","), "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
+               "order": args.order.split(",") if args.design == "gogudra" else None, "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
         steps, warmup = min(args.steps, 64), min(args.warmup, 4)
         for name in ("qwen25vl", args.design):
             if name != "qwen25vl":
                 del model
                 torch.cuda.empty_cache()
-                model = build_model(load_config(gogudra_config(args.layers, args.size, tuple(args.order.split(",")))),
-                                    dtype, "cuda:0")
+                design = (dazapel_config(args.layers, args.size) if args.design == "dazapel"
+                          else gogudra_config(args.layers, args.size, tuple(args.order.split(","))))
+                model = build_model(load_config(design), dtype, "cuda:0")
                 fill_random(model, seed=0)
                 torch.cuda.synchronize()
             sec = prefill_rate(2048)

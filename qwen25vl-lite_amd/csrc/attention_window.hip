@@ -109,8 +109,12 @@ __global__ __launch_bounds__(256) void attn_window_kernel(WindowArgs a) {
       s[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
+        // no load inside a branch (the compiler would wait for each before the next): channels past the
+        // head's end are read from its start and replaced by zeros
         const int d = ks * 32 + 8 * lg;
-        const bf16x8_t kf = d < HD ? load8(krow + d) : zero8();
+        const bool d_ok = (HD % 32 == 0) || d < HD;
+        bf16x8_t kf = load8(krow + (d_ok ? d : 0));
+        kf = d_ok ? kf : zero8();
         s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qb[ks], s[t], 0, 0, 0);
       }
     }
@@ -153,7 +157,9 @@ __global__ __launch_bounds__(256) void attn_window_kernel(WindowArgs a) {
 #pragma unroll
     for (int dt = 0; dt < NT; ++dt) {
       const int c = dt * 16 + r;
-      const bf16x8_t vf = c < VD ? load8(vbase + (size_t)c * a.ps) : zero8();
+      const bool c_ok = (VD % 16 == 0) || c < VD;
+      bf16x8_t vf = load8(vbase + (size_t)(c_ok ? c : 0) * a.ps);
+      vf = c_ok ? vf : zero8();
       acc[dt] *= alpha;
       acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, acc[dt], 0, 0, 0);
     }

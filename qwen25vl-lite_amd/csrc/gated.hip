@@ -455,35 +455,35 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
   __shared__ float red[17];
   const int m = blockIdx.x, n = rows ? rows[m] : m;
   float* hr = h + (size_t)n * H;
-  float val[SN_VPT];
-  float rs = 1.0f;
-  if (y) {
-    const TY* yr = y + (size_t)n * H;
-    float ss = 0.f;
+  // Everything a thread needs of the row is asked for before the first sum is waited for, and no load
+  // stands inside a branch (the compiler would wait for each before the next): a column past the row's
+  // end reads column 0 and counts as zero.
+  float val[SN_VPT], hv[SN_VPT], gv[SN_VPT], wv[SN_VPT];
+  float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < SN_VPT; ++i) {
-      const int c = threadIdx.x + i * blockDim.x;
-      float v = 0.f;
-      if (c < H) {
-        v = ldf<TY>(yr + c);
-        for (int s = 1; s < nslabs; ++s) v += ldf<TY>(yr + (size_t)s * slab_stride + c);
-      }
-      val[i] = v;
-      ss += v * v;
-    }
-    if (gain) rs = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps_y);
+  for (int i = 0; i < SN_VPT; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    const bool ok = c < H;
+    const int cc = ok ? c : 0;
+    float v = y ? ldf<TY>(y + (size_t)n * H + cc) : 0.f;
+    for (int s = 1; s < nslabs; ++s) v += ldf<TY>(y + (size_t)s * slab_stride + (size_t)n * H + cc);
+    float add = vec ? vec[cc] : 0.f;
+    hv[i] = ok ? hr[cc] + add : 0.f;
+    gv[i] = gain ? gain[cc] : 1.f;
+    wv[i] = w ? w[cc] : 1.f;
+    v = ok ? v : 0.f;
+    val[i] = v;
+    ss += v * v;
   }
+  float rs = 1.0f;
+  if (y && gain) rs = factor / sqrtf(block_sum(ss, red) / (float)H + eps_y);
   float ss2 = 0.f;
 #pragma unroll
   for (int i = 0; i < SN_VPT; ++i) {
     const int c = threadIdx.x + i * blockDim.x;
-    float v = 0.f;
-    if (c < H) {
-      v = hr[c];
-      if (y) v += gain ? factor * ((val[i] * rs) * gain[c]) : val[i];
-      if (vec) v += vec[c];
-      if (!rows && (y || vec)) hr[c] = v;
-    }
+    float v = hv[i];
+    if (y) v += gain ? (val[i] * rs) * gv[i] : val[i];
+    if (c < H && !rows && (y || vec)) hr[c] = v;
     val[i] = v;
     ss2 += v * v;
   }
@@ -493,7 +493,7 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
 #pragma unroll
   for (int i = 0; i < SN_VPT; ++i) {
     const int c = threadIdx.x + i * blockDim.x;
-    if (c < H) stf<TO>(o + c, (val[i] * rs2) * w[c]);
+    if (c < H) stf<TO>(o + c, (val[i] * rs2) * wv[i]);
   }
 }
 

@@ -216,7 +216,8 @@ __global__ __launch_bounds__(256) void moe_rows_kernel(ExpertArgs a) {
   }
 }
 
-// bfloat16 on the matrix cores.  A block of four waves owns 16 MT pairs of one expert and 64 output
+// bfloat16 on the matrix cores, few pairs an expert (a decode step: the experts' weights are read once
+// each and that is the time it takes).  A block of four waves owns 16 MT pairs of one expert and 64 output
 // columns; a wave takes 16 of the columns (rows of W: the instruction's first operand, straight from
 // memory: nobody else in the block reads them) and all MT tiles of 16 pairs (rows of x: the second
 // operand).  K in steps of 32, a multiple of 8.  Which expert a block serves follows from the
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
   const bf16_t* we = (const bf16_t*)a.w + (size_t)e * rows_w * a.K;
   const bool col_ok = c0 + r < a.R;
   const bf16_t* wg = we + (size_t)(col_ok ? c0 + r : 0) * a.K + 8 * lg;
-  const bf16_t* wu = wg + (size_t)a.R * a.K;
+  const bf16_t* wu = wg + (size_t)a.R * a.K;      // only read if gated
   const bf16_t* xr[MT];
   int pair[MT];
 #pragma unroll
@@ -256,17 +257,26 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
     accg[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     accu[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
+  // No load stands inside a branch (the compiler would wait for each before the next): what does not
+  // exist is read from a place that does (column 0 of the step, row 0) and replaced by zeros.
   const bf16x8_t zero = __builtin_bit_cast(bf16x8_t, uint4{0u, 0u, 0u, 0u});
+  if (!a.gated) wu = wg;
+#pragma unroll 2
   for (int k = 0; k < a.K; k += 32) {
     const bool k_ok = k + 8 * lg < a.K;
-    const bf16x8_t fg = (k_ok && col_ok) ? *reinterpret_cast<const bf16x8_t*>(wg + k) : zero;
-    bf16x8_t fu = zero;
-    if (a.gated && k_ok && col_ok) fu = *reinterpret_cast<const bf16x8_t*>(wu + k);
+    const int at = k_ok ? k : k - 8 * lg;
+    bf16x8_t fg = *reinterpret_cast<const bf16x8_t*>(wg + at);
+    bf16x8_t fu = *reinterpret_cast<const bf16x8_t*>(wu + at);
+    bf16x8_t fx[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) fx[t] = *reinterpret_cast<const bf16x8_t*>(xr[t] + at);
+    fg = (k_ok && col_ok) ? fg : zero;
+    fu = (k_ok && col_ok) ? fu : zero;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      const bf16x8_t fx = (k_ok && pair[t] >= 0) ? *reinterpret_cast<const bf16x8_t*>(xr[t] + k) : zero;
-      accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg, fx, accg[t], 0, 0, 0);
-      if (a.gated) accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu, fx, accu[t], 0, 0, 0);
+      const bf16x8_t f = (k_ok && pair[t] >= 0) ? fx[t] : zero;
+      accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg, f, accg[t], 0, 0, 0);
+      if (a.gated) accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu, f, accu[t], 0, 0, 0);
     }
   }
   // a lane holds, of tile t, pair r and columns c0 + 4 lg .. + 3
@@ -284,9 +294,181 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
   }
 }
 
+// Many pairs an expert: tiles of 128 pairs x 128 rows of W (gated: 64 gate rows and the 64 up rows of the
+// same outputs), K in steps of TILE_K through LDS.  The 256 threads fetch the next step's 128 x TILE_K values
+// of x (gathered rows) and of W into registers while the step in LDS is multiplied, then put them into
+// the other of two buffers; the 16-byte chunks of a row are exchanged by bits of the row number, so that
+// the 16 lanes that read one chunk of 16 rows hit all 64 banks.  The four
+// waves stand 2 x 2: each owns 64 pairs and 64 rows of W (gated: 32 gate rows and their 32 up rows),
+// 16 products of 16 x 16 x 32 a step from 8 operand reads.
+#define TILE_M 128
+#define TILE_N 128
+#ifndef TILE_K
+#define TILE_K 64
+#endif
+#ifndef MOE_PROBE
+#define MOE_PROBE 0
+#endif
+#ifndef MOE_ORDER
+#define MOE_ORDER 2
+#endif
+#define ROW_CHUNKS (TILE_K / 8)                        // 16-byte chunks of a row of a tile
+#define THREAD_CHUNKS (TILE_M * ROW_CHUNKS / 256)      // chunks of x (and of W) a thread fetches a step
+
+__device__ __forceinline__ int lds_slot(int row, int chunk) {
+#if TILE_K == 64
+  return row * 8 + (chunk ^ ((row >> 1) & 7));
+#else
+  return row * 4 + (chunk ^ ((row >> 2) & 3));
+#endif
+}
+
+template <bool GATED, typename TO>
+__global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m, int tiles_n) {
+  __shared__ __attribute__((aligned(16))) uint4 s_x[2][TILE_M * ROW_CHUNKS];
+  __shared__ __attribute__((aligned(16))) uint4 s_w[2][TILE_N * ROW_CHUNKS];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+#if MOE_ORDER == 2
+  // Blocks go to the XCDs in turn (block b to XCD b mod 8, each with an L2 of its own).  The 32 blocks that
+  // an XCD's compute units hold at a time are made 4 tiles of pairs x 8 tiles of rows of W: they walk K at
+  // about the same pace, so a slice of x is fetched into that L2 once for 8 blocks and a slice of W once for 4.
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int super = (idx >> 5) * 8 + xcd, inner = idx & 31;
+  const int supers_m = (tiles_m + 3) / 4;
+  const int tile_n = (super / supers_m) * 8 + (inner >> 2);
+  int tile = (super % supers_m) * 4 + (inner & 3);
+  if (tile >= tiles_m || tile_n >= tiles_n) return;
+#elif MOE_ORDER == 1
+  const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
+  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (work >= total) return;
+  int tile = work % tiles_m;
+  const int tile_n = work / tiles_m;
+#else
+  int tile = blockIdx.x % tiles_m;
+  const int tile_n = blockIdx.x / tiles_m;
+#endif
+  int e = 0, first = 0, last = 0;
+  for (; e < a.E; ++e) {
+    first = a.offsets[e];
+    last = a.offsets[e + 1];
+    const int nt = (last - first + TILE_M - 1) / TILE_M;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (e >= a.E) return;
+  first += tile * TILE_M;
+  constexpr int OUT_COLS = GATED ? TILE_N / 2 : TILE_N;     // output columns of a block
+  const int c0 = tile_n * OUT_COLS;
+  const int rows_w = GATED ? 2 * a.R : a.R;
+  const bf16_t* we = (const bf16_t*)a.w + (size_t)e * rows_w * a.K;
+
+  // what this thread fetches each step: chunks of 16 bytes of x and as many of W
+  const bf16_t* gx[THREAD_CHUNKS];
+  const bf16_t* gw[THREAD_CHUNKS];
+  bool x_ok[THREAD_CHUNKS], w_ok[THREAD_CHUNKS];
+  int slot[THREAD_CHUNKS];
+#pragma unroll
+  for (int j = 0; j < THREAD_CHUNKS; ++j) {
+    const int id = threadIdx.x + 256 * j, row = id / ROW_CHUNKS, ch = id % ROW_CHUNKS;
+    slot[j] = lds_slot(row, ch);
+    const int i = first + row;
+    const int pair = i < last ? a.sorted[i] : -1;
+    x_ok[j] = pair >= 0;
+    gx[j] = (const bf16_t*)a.x + (size_t)(pair < 0 ? 0 : pair / a.div) * a.ldx + 8 * ch;
+    int wrow;                                               // row of W_e behind row `row` of the tile
+    if (GATED) wrow = row < 64 ? c0 + row : a.R + c0 + (row - 64);
+    else wrow = c0 + row;
+    const bool ok = GATED ? (c0 + (row & 63) < a.R) : (wrow < a.R);
+    w_ok[j] = ok;
+    gw[j] = we + (size_t)(ok ? wrow : 0) * a.K + 8 * ch;
+  }
+  // No load stands inside a branch (the compiler would wait for each before the next): a chunk that
+  // does not exist is read from one that does (row 0, column 0 of the step) and replaced by zeros.
+  const uint4 zero = uint4{0u, 0u, 0u, 0u};
+  uint4 rx[THREAD_CHUNKS], rw[THREAD_CHUNKS];
+  auto fetch = [&](int k) {
+#pragma unroll
+    for (int j = 0; j < THREAD_CHUNKS; ++j) {
+      const int ch = (threadIdx.x + 256 * j) % ROW_CHUNKS;
+      const bool k_ok = k + 8 * ch < a.K;
+      const int at = k_ok ? k : k - 8 * ch;
+      const uint4 vx = *reinterpret_cast<const uint4*>(gx[j] + at);
+      const uint4 vw = *reinterpret_cast<const uint4*>(gw[j] + at);
+      const bool fx_ok = x_ok[j] && k_ok, fw_ok = w_ok[j] && k_ok;
+      rx[j] = uint4{fx_ok ? vx.x : 0u, fx_ok ? vx.y : 0u, fx_ok ? vx.z : 0u, fx_ok ? vx.w : 0u};
+      rw[j] = uint4{fw_ok ? vw.x : 0u, fw_ok ? vw.y : 0u, fw_ok ? vw.z : 0u, fw_ok ? vw.w : 0u};
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < THREAD_CHUNKS; ++j) {
+      s_x[buf][slot[j]] = rx[j];
+      s_w[buf][slot[j]] = rw[j];
+    }
+  };
+  f32x4_t acc[4][4];     // [tile of 16 rows of W][tile of 16 pairs]
+#pragma unroll
+  for (int n = 0; n < 4; ++n)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[n][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  // rows of the W tile this wave multiplies: gated, 32 gate rows and the 32 up rows of the same outputs
+  int wrow0[4];
+#pragma unroll
+  for (int n = 0; n < 4; ++n) wrow0[n] = GATED ? (n < 2 ? wn * 32 + n * 16 : 64 + wn * 32 + (n - 2) * 16) : wn * 64 + n * 16;
+
+  fetch(0);
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k = 0; k < a.K; k += TILE_K) {
+    const bool more = k + TILE_K < a.K;
+#if MOE_PROBE != 1
+    if (more) fetch(k + TILE_K);
+#endif
+#if MOE_PROBE != 2
+#pragma unroll
+    for (int kk = 0; kk < TILE_K / 32; ++kk) {
+      bf16x8_t fw[4], fx[4];
+#pragma unroll
+      for (int n = 0; n < 4; ++n) fw[n] = __builtin_bit_cast(bf16x8_t, s_w[buf][lds_slot(wrow0[n] + r, 4 * kk + lg)]);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) fx[m] = __builtin_bit_cast(bf16x8_t, s_x[buf][lds_slot(wm * 64 + m * 16 + r, 4 * kk + lg)]);
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[n][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[n], fx[m], acc[n][m], 0, 0, 0);
+    }
+#endif
+    if (more) put(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+  // a lane holds, of (n, m): pair wm 64 + 16 m + r, W rows wrow0[n] + 4 lg .. + 3
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const int i = first + wm * 64 + m * 16 + r;
+    if (i >= last) continue;
+    const int pair = a.sorted[i];
+    TO* o = (TO*)a.out + (size_t)pair * a.R;
+#pragma unroll
+    for (int n = 0; n < (GATED ? 2 : 4); ++n) {
+      const int c = c0 + (GATED ? wn * 32 + n * 16 : wn * 64 + n * 16) + 4 * lg;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (c + j >= a.R) break;
+        float v = acc[n][m][j];
+        if (GATED) v = gated_value(v, acc[n + 2][m][j], a.alpha, a.limit, a.shift);
+        stf<TO>(o + c + j, v);
+      }
+    }
+  }
+}
+
 // x_dtype / out_dtype: 0 float32, 1 bfloat16.  float32 operands write float32; bfloat16 operands
 // write either.  The matrix-core kernel runs for bfloat16 with K a multiple of 8 and rows of x on
-// 16-byte boundaries; `big_tiles` asks for tiles of 64 pairs instead of 16 (many pairs an expert).
+// 16-byte boundaries; `big_tiles` asks for the kernel with tiles of 128 pairs through LDS (many pairs an expert).
 extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const void* w, const void* sorted,
                                const void* offsets, void* out, int out_dtype, int P, int E, int R, int K, int div,
                                int gated, float alpha, float limit, float shift, int big_tiles, hipStream_t stream) {
@@ -296,13 +478,26 @@ extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const 
   a.x = x; a.ldx = ldx; a.w = w; a.sorted = (const int*)sorted; a.offsets = (const int*)offsets; a.out = out;
   a.P = P; a.E = E; a.R = R; a.K = K; a.div = div; a.gated = gated; a.alpha = alpha; a.limit = limit; a.shift = shift;
   if (x_dtype == 1 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0) {
-    const int tm = big_tiles ? 64 : 16;
-    const int tiles = P / tm + (E < P ? E : P);
+    if (out_dtype != 0 && out_dtype != 1) return QVL_ERR_DTYPE;
+    if (big_tiles) {
+      const int cols = gated ? TILE_N / 2 : TILE_N;
+      const int tiles_m = P / TILE_M + (E < P ? E : P), tiles_n = (R + cols - 1) / cols;
+      if ((long long)tiles_m * tiles_n > 0x7ffffff0ll) return QVL_ERR_LIMIT;
+      // whole groups of 4 x 8 tiles, 8 groups (one per XCD) at a time
+      const int supers = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
+      const dim3 tgrid((unsigned)((supers + 7) / 8) * 8 * 32);
+      if (gated && out_dtype == 1)
+        hipLaunchKernelGGL((moe_tile_kernel<true, bf16_t>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      else if (gated) hipLaunchKernelGGL((moe_tile_kernel<true, float>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      else if (out_dtype == 1)
+        hipLaunchKernelGGL((moe_tile_kernel<false, bf16_t>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      else hipLaunchKernelGGL((moe_tile_kernel<false, float>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      return qvl_launch_status();
+    }
+    const int tiles = P / 16 + (E < P ? E : P);
     const dim3 grid(tiles, (R + 63) / 64);
     if (grid.y > 65535) return QVL_ERR_LIMIT;
-    if (big_tiles && out_dtype == 1) hipLaunchKernelGGL((moe_mfma_kernel<4, bf16_t>), grid, dim3(256), 0, stream, a);
-    else if (big_tiles && out_dtype == 0) hipLaunchKernelGGL((moe_mfma_kernel<4, float>), grid, dim3(256), 0, stream, a);
-    else if (out_dtype == 1) hipLaunchKernelGGL((moe_mfma_kernel<1, bf16_t>), grid, dim3(256), 0, stream, a);
+    if (out_dtype == 1) hipLaunchKernelGGL((moe_mfma_kernel<1, bf16_t>), grid, dim3(256), 0, stream, a);
     else if (out_dtype == 0) hipLaunchKernelGGL((moe_mfma_kernel<1, float>), grid, dim3(256), 0, stream, a);
     else return QVL_ERR_DTYPE;
     return qvl_launch_status();
@@ -322,20 +517,23 @@ extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const 
 // a shared expert gave: float32 or bfloat16, or float32 slabs added in order; null: nothing).
 // ---------------------------------------------------------------------------------------
 template <typename TY, typename TX>
-__global__ void moe_combine_kernel(const TY* __restrict__ y, const float* __restrict__ wts, const TX* __restrict__ extra,
-                                   int nslabs, long long slab_stride, float* __restrict__ out, int top, int H) {
+__global__ __launch_bounds__(256) void moe_combine_kernel(const TY* __restrict__ y, const float* __restrict__ wts,
+                                                          const TX* __restrict__ extra, int nslabs, long long slab_stride,
+                                                          float* __restrict__ out, int top, int H) {
+  // a thread owns one column of one token: its loads are all on their way before the first is used
   const size_t n = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= H) return;
   const float* wr = wts + n * top;
-  for (int c = threadIdx.x; c < H; c += blockDim.x) {
-    float v = 0.f;
-    for (int k = 0; k < top; ++k) v += wr[k] * ldf<TY>(y + (n * top + k) * (size_t)H + c);
-    if (extra) {
-      float x = ldf<TX>(extra + n * H + c);
-      for (int s = 1; s < nslabs; ++s) x += ldf<TX>(extra + (size_t)s * slab_stride + n * H + c);
-      v += x;
-    }
-    out[n * H + c] = v;
+  float v = 0.f;
+#pragma unroll 8
+  for (int k = 0; k < top; ++k) v += wr[k] * ldf<TY>(y + (n * top + k) * (size_t)H + c);
+  if (extra) {
+    float x = ldf<TX>(extra + n * H + c);
+    for (int s = 1; s < nslabs; ++s) x += ldf<TX>(extra + (size_t)s * slab_stride + n * H + c);
+    v += x;
   }
+  out[n * H + c] = v;
 }
 
 extern "C" int qvl_moe_combine(const void* y, int y_dtype, const void* wts, const void* extra, int extra_dtype,
@@ -343,7 +541,8 @@ extern "C" int qvl_moe_combine(const void* y, int y_dtype, const void* wts, cons
   if (N <= 0) return QVL_OK;
   if (top <= 0 || H <= 0 || nslabs < 1 || (nslabs > 1 && extra_dtype != 0)) return QVL_ERR_SHAPE;
 #define LAUNCH(TY, TX)                                                                                         \
-  hipLaunchKernelGGL((moe_combine_kernel<TY, TX>), dim3(N), dim3(256), 0, stream, (const TY*)y, (const float*)wts, \
+  hipLaunchKernelGGL((moe_combine_kernel<TY, TX>), dim3(N, (H + 255) / 256), dim3(256), 0, stream, (const TY*)y,   \
+                     (const float*)wts,                                                                            \
                      (const TX*)extra, nslabs, slab_stride, (float*)out, top, H)
   if (y_dtype == 0 && extra_dtype == 0) LAUNCH(float, float);
   else if (y_dtype == 0 && extra_dtype == 1) LAUNCH(float, bf16_t);

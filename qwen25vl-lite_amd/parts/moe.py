@@ -21,6 +21,8 @@ from .base import FeedForward, ParamSpec, Part, PartSpec, StepContext, build_par
 
 __all__ = ["RoutedExperts"]
 
+FLOAT32_PAIRS = 512     # up to this many (token, expert) pairs the experts' results stay float32 until they are summed
+
 
 class RoutedExperts(FeedForward):
     """params: ``hidden_size``, ``num_experts``, ``top``, ``intermediate_size`` (of one expert),
@@ -116,7 +118,9 @@ class RoutedExperts(FeedForward):
         pairs = n * self.top
         act = moe_ops.expert_products(x, self.w_gate_up, order, offsets, pairs, self.top, self.dtype,
                                       gated=(self.alpha, self.limit, self.shift))
-        y = moe_ops.expert_products(act, self.w_down, order, offsets, pairs, 1, torch.float32)
+        # few pairs: the float32 sums as they are; many: one rounding, half the traffic
+        y = moe_ops.expert_products(act, self.w_down, order, offsets, pairs, 1,
+                                    torch.float32 if pairs <= FLOAT32_PAIRS else self.dtype)
         extra = None
         if self.shared is not None:
             residual, step.residual = step.residual, None      # the shared expert's result is an addend of this sum

@@ -145,9 +145,9 @@ def test_router(e, top, groups, keep):
 
 @pytest.mark.parametrize("dtype, width, ff", [(torch.float32, 56, 24), (torch.bfloat16, 64, 40), (torch.bfloat16, 56, 24),
                                               (torch.bfloat16, 50, 11), (torch.float32, 50, 11)])
-@pytest.mark.parametrize("rows", [3, 150])
+@pytest.mark.parametrize("rows", [3, 150, 700])
 def test_routed_experts_alone(dtype, width, ff, rows, tmp_path):
-    """Few rows (a tile of 16 pairs an expert) and many (tiles of 64), widths on and off the matrix
+    """Few rows (a tile of 16 pairs an expert) and many (one and several tiles of 128), widths on and off the matrix
     cores' steps, in float32 and bfloat16, with a shared expert and clamps that bite."""
     mlp = du.moe(6, 3, ff, 0.8, groups=(3, 2), scale=1.3, shared=(ff + 8, 0.5))
     lay = du.layer(du.attention(1, 1, 16, 16, 16, scale=0.25), mlp)
@@ -155,7 +155,7 @@ def test_routed_experts_alone(dtype, width, ff, rows, tmp_path):
     torch.manual_seed(rows)
     x = torch.randn(rows, width).to(dtype)
     want = plain.moe(x.double(), t, "l0.mlp.", mlp)
-    step = _step_for(runner, "a", rows) if rows <= 256 else None
+    step = _step_for(runner, "a", min(rows, 256))
     got = block.ffn.forward(x.cuda(), step).double().cpu()
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     assert torch.allclose(got, want, atol=tol * want.abs().max().item()), (got - want).abs().max()
@@ -218,7 +218,7 @@ def test_float32_every_schedule_against_the_plain_model(name, folders):
     assert any(len(who) > 1 for who in holders.values()), "no page was used by two requests"
 
 
-@pytest.mark.parametrize("name", ["mixed", "ones"])
+@pytest.mark.parametrize("name", ["mixed", "ones", "odd"])
 def test_bfloat16_within_rounding_of_the_plain_model(name, folders):
     """bfloat16 kernels: no further from exact arithmetic than rounding the stored activations to
     bfloat16 takes the plain model, whatever the schedule."""
