@@ -43,16 +43,21 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
           and block_table.shape[0] == step.num_reqs, "block_table must be int32 [R, width]")
     _need(nq % nkv == 0, "query heads must be a multiple of key/value heads")
     group = nq // nkv
+    defines = {"HD": hd, "VD": vd}
     tile_req, tile_ct, num_tiles = _step_tiles(step, group, 1, q.device)
-    cu_q = step.cu_q
-    if step.max_q_len == 1 and num_tiles == step.num_reqs == len(step.cu_q_host) - 1 == step.cu_q_host[-1]:
-        tile_req = tile_ct = cu_q = None     # decoded tokens only: request i brings token i and has tile i
     if share is None:
         share = num_tiles * nkv < SHARE_BELOW_PER_CU * _compute_units(q.device)
+    cu_q = step.cu_q
+    if share and step.max_q_len == 1 and num_tiles == step.num_reqs == len(step.cu_q_host) - 1 == step.cu_q_host[-1]:
+        tile_req = tile_ct = cu_q = None     # decoded tokens only: request i brings token i and has tile i
+    elif not share:
+        # a wave owns an entry of several neighbouring column tiles
+        wide = int(_fn("attention_window", "qvl_attn_window_entry_tiles", [], defines)())
+        tile_req, tile_ct, num_tiles = _step_tiles(step, group, wide, q.device)
     out = torch.empty((n, nq * vd), dtype=q.dtype, device=q.device)
     fn = _fn("attention_window", "qvl_attn_window",
              [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 5 + [_c_float, _c_int, _c_ptr],
-             {"HD": hd, "VD": vd})
+             defines)
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(cu_q),
               _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), nq, nkv, ps, int(window or 0),
               int(keep_first) if window else 0, float(scale), int(bool(share)), _stream()),
