@@ -294,26 +294,28 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
   }
 }
 
-// Many pairs an expert: tiles of 128 pairs x 128 rows of W (gated: 64 gate rows and the 64 up rows of the
-// same outputs), K in steps of TILE_K through LDS.  The 256 threads fetch the next step's 128 x TILE_K values
-// of x (gathered rows) and of W into registers while the step in LDS is multiplied, then put them into
-// the other of two buffers; the 16-byte chunks of a row are exchanged by bits of the row number, so that
-// the 16 lanes that read one chunk of 16 rows hit all 64 banks.  The four
-// waves stand 2 x 2: each owns 64 pairs and 64 rows of W (gated: 32 gate rows and their 32 up rows),
-// 16 products of 16 x 16 x 32 a step from 8 operand reads.
-#define TILE_M 128
-#define TILE_N 128
+// Many pairs an expert: tiles of TILE_M pairs x TILE_N rows of W (gated: TILE_N / 2 gate rows and the up rows
+// of the same outputs), K in steps of TILE_K through LDS.  The 256 threads fetch the next step's values of x
+// (gathered rows) and of W into registers while the step in LDS is multiplied, then put them into the other
+// of two buffers; the 16-byte chunks of a row are exchanged by bits of the row number, so that the 16 lanes
+// that read one chunk of 16 rows hit all 64 banks.  The four waves stand 2 x 2: each owns 64 pairs and
+// 16 NW rows of W (gated: 8 NW gate rows and their up rows): 4 NW products of 16 x 16 x 32 a step from
+// 4 + NW operand reads.
+// Measured on 12,288 pairs over 32 experts, K 3,584, 2 x 2,368 rows (gate|up): TILE_K 64, NW 4: 1,000 us; TILE_K 32:
+// 1,030; NW 8 (tiles of 128 x 256: fewer operand reads and fetched bytes a product, but the sums leave
+// room for one wave a SIMD): 1,220 (TILE_K 64), 1,420 (TILE_K 32); fetching two steps ahead into a
+// second set of registers: 1,230.
 #ifndef TILE_K
 #define TILE_K 64
 #endif
-#ifndef MOE_PROBE
-#define MOE_PROBE 0
+#ifndef NW
+#define NW 4                                           // tiles of 16 rows of W a wave multiplies
 #endif
-#ifndef MOE_ORDER
-#define MOE_ORDER 2
-#endif
+#define TILE_M 128
+#define TILE_N (32 * NW)
 #define ROW_CHUNKS (TILE_K / 8)                        // 16-byte chunks of a row of a tile
-#define THREAD_CHUNKS (TILE_M * ROW_CHUNKS / 256)      // chunks of x (and of W) a thread fetches a step
+#define X_CHUNKS (TILE_M * ROW_CHUNKS / 256)           // chunks of x a thread fetches a step
+#define W_CHUNKS (TILE_N * ROW_CHUNKS / 256)           // and of W
 
 __device__ __forceinline__ int lds_slot(int row, int chunk) {
 #if TILE_K == 64
@@ -329,7 +331,6 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
   __shared__ __attribute__((aligned(16))) uint4 s_w[2][TILE_N * ROW_CHUNKS];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
   const int wm = wave >> 1, wn = wave & 1;
-#if MOE_ORDER == 2
   // Blocks go to the XCDs in turn (block b to XCD b mod 8, each with an L2 of its own).  The 32 blocks that
   // an XCD's compute units hold at a time are made 4 tiles of pairs x 8 tiles of rows of W: they walk K at
   // about the same pace, so a slice of x is fetched into that L2 once for 8 blocks and a slice of W once for 4.
@@ -339,16 +340,6 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
   const int tile_n = (super / supers_m) * 8 + (inner >> 2);
   int tile = (super % supers_m) * 4 + (inner & 3);
   if (tile >= tiles_m || tile_n >= tiles_n) return;
-#elif MOE_ORDER == 1
-  const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (work >= total) return;
-  int tile = work % tiles_m;
-  const int tile_n = work / tiles_m;
-#else
-  int tile = blockIdx.x % tiles_m;
-  const int tile_n = blockIdx.x / tiles_m;
-#endif
   int e = 0, first = 0, last = 0;
   for (; e < a.E; ++e) {
     first = a.offsets[e];
@@ -359,64 +350,76 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
   }
   if (e >= a.E) return;
   first += tile * TILE_M;
-  constexpr int OUT_COLS = GATED ? TILE_N / 2 : TILE_N;     // output columns of a block
+  constexpr int HALF = TILE_N / 2;
+  constexpr int OUT_COLS = GATED ? HALF : TILE_N;           // output columns of a block
   const int c0 = tile_n * OUT_COLS;
   const int rows_w = GATED ? 2 * a.R : a.R;
   const bf16_t* we = (const bf16_t*)a.w + (size_t)e * rows_w * a.K;
 
-  // what this thread fetches each step: chunks of 16 bytes of x and as many of W
-  const bf16_t* gx[THREAD_CHUNKS];
-  const bf16_t* gw[THREAD_CHUNKS];
-  bool x_ok[THREAD_CHUNKS], w_ok[THREAD_CHUNKS];
-  int slot[THREAD_CHUNKS];
+  // what this thread fetches each step: chunks of 16 bytes of x and of W.  No load stands inside a branch
+  // (the compiler would wait for each before the next): a chunk that does not exist is read from one
+  // that does (row 0, column 0 of the step) and replaced by zeros.
+  const bf16_t* gx[X_CHUNKS];
+  const bf16_t* gw[W_CHUNKS];
+  bool x_ok[X_CHUNKS], w_ok[W_CHUNKS];
 #pragma unroll
-  for (int j = 0; j < THREAD_CHUNKS; ++j) {
+  for (int j = 0; j < X_CHUNKS; ++j) {
     const int id = threadIdx.x + 256 * j, row = id / ROW_CHUNKS, ch = id % ROW_CHUNKS;
-    slot[j] = lds_slot(row, ch);
     const int i = first + row;
     const int pair = i < last ? a.sorted[i] : -1;
     x_ok[j] = pair >= 0;
     gx[j] = (const bf16_t*)a.x + (size_t)(pair < 0 ? 0 : pair / a.div) * a.ldx + 8 * ch;
-    int wrow;                                               // row of W_e behind row `row` of the tile
-    if (GATED) wrow = row < 64 ? c0 + row : a.R + c0 + (row - 64);
-    else wrow = c0 + row;
-    const bool ok = GATED ? (c0 + (row & 63) < a.R) : (wrow < a.R);
-    w_ok[j] = ok;
-    gw[j] = we + (size_t)(ok ? wrow : 0) * a.K + 8 * ch;
   }
-  // No load stands inside a branch (the compiler would wait for each before the next): a chunk that
-  // does not exist is read from one that does (row 0, column 0 of the step) and replaced by zeros.
-  const uint4 zero = uint4{0u, 0u, 0u, 0u};
-  uint4 rx[THREAD_CHUNKS], rw[THREAD_CHUNKS];
-  auto fetch = [&](int k) {
 #pragma unroll
-    for (int j = 0; j < THREAD_CHUNKS; ++j) {
-      const int ch = (threadIdx.x + 256 * j) % ROW_CHUNKS;
-      const bool k_ok = k + 8 * ch < a.K;
-      const int at = k_ok ? k : k - 8 * ch;
-      const uint4 vx = *reinterpret_cast<const uint4*>(gx[j] + at);
-      const uint4 vw = *reinterpret_cast<const uint4*>(gw[j] + at);
-      const bool fx_ok = x_ok[j] && k_ok, fw_ok = w_ok[j] && k_ok;
-      rx[j] = uint4{fx_ok ? vx.x : 0u, fx_ok ? vx.y : 0u, fx_ok ? vx.z : 0u, fx_ok ? vx.w : 0u};
-      rw[j] = uint4{fw_ok ? vw.x : 0u, fw_ok ? vw.y : 0u, fw_ok ? vw.z : 0u, fw_ok ? vw.w : 0u};
+  for (int j = 0; j < W_CHUNKS; ++j) {
+    const int id = threadIdx.x + 256 * j, row = id / ROW_CHUNKS, ch = id % ROW_CHUNKS;
+    int wrow;                                               // row of W_e behind row `row` of the tile
+    if (GATED) wrow = row < HALF ? c0 + row : a.R + c0 + (row - HALF);
+    else wrow = c0 + row;
+    w_ok[j] = GATED ? (c0 + (row % HALF) < a.R) : (wrow < a.R);
+    gw[j] = we + (size_t)(w_ok[j] ? wrow : 0) * a.K + 8 * ch;
+  }
+  uint4 rx[X_CHUNKS], rw[W_CHUNKS];
+  auto fetch = [&](int k) {
+    const int ch = threadIdx.x % ROW_CHUNKS;                // 256 is a multiple of ROW_CHUNKS: the same for every j
+    const bool k_ok = k + 8 * ch < a.K;
+    const int at = k_ok ? k : k - 8 * ch;
+#pragma unroll
+    for (int j = 0; j < X_CHUNKS; ++j) {
+      const uint4 v = *reinterpret_cast<const uint4*>(gx[j] + at);
+      const bool ok = x_ok[j] && k_ok;
+      rx[j] = uint4{ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u};
+    }
+#pragma unroll
+    for (int j = 0; j < W_CHUNKS; ++j) {
+      const uint4 v = *reinterpret_cast<const uint4*>(gw[j] + at);
+      const bool ok = w_ok[j] && k_ok;
+      rw[j] = uint4{ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u};
     }
   };
   auto put = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < THREAD_CHUNKS; ++j) {
-      s_x[buf][slot[j]] = rx[j];
-      s_w[buf][slot[j]] = rw[j];
+    for (int j = 0; j < X_CHUNKS; ++j) {
+      const int id = threadIdx.x + 256 * j;
+      s_x[buf][lds_slot(id / ROW_CHUNKS, id % ROW_CHUNKS)] = rx[j];
+    }
+#pragma unroll
+    for (int j = 0; j < W_CHUNKS; ++j) {
+      const int id = threadIdx.x + 256 * j;
+      s_w[buf][lds_slot(id / ROW_CHUNKS, id % ROW_CHUNKS)] = rw[j];
     }
   };
-  f32x4_t acc[4][4];     // [tile of 16 rows of W][tile of 16 pairs]
+  f32x4_t acc[NW][4];    // [tile of 16 rows of W][tile of 16 pairs]
 #pragma unroll
-  for (int n = 0; n < 4; ++n)
+  for (int n = 0; n < NW; ++n)
 #pragma unroll
     for (int m = 0; m < 4; ++m) acc[n][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  // rows of the W tile this wave multiplies: gated, 32 gate rows and the 32 up rows of the same outputs
-  int wrow0[4];
+  // rows of the W tile this wave multiplies: gated, its gate rows and the up rows of the same outputs
+  constexpr int PER_WAVE = GATED ? 8 * NW : 16 * NW;        // output columns of a wave
+  int wrow0[NW];
 #pragma unroll
-  for (int n = 0; n < 4; ++n) wrow0[n] = GATED ? (n < 2 ? wn * 32 + n * 16 : 64 + wn * 32 + (n - 2) * 16) : wn * 64 + n * 16;
+  for (int n = 0; n < NW; ++n)
+    wrow0[n] = GATED ? (n < NW / 2 ? wn * PER_WAVE + n * 16 : HALF + wn * PER_WAVE + (n - NW / 2) * 16) : wn * PER_WAVE + n * 16;
 
   fetch(0);
   put(0);
@@ -424,23 +427,19 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
   int buf = 0;
   for (int k = 0; k < a.K; k += TILE_K) {
     const bool more = k + TILE_K < a.K;
-#if MOE_PROBE != 1
     if (more) fetch(k + TILE_K);
-#endif
-#if MOE_PROBE != 2
 #pragma unroll
     for (int kk = 0; kk < TILE_K / 32; ++kk) {
-      bf16x8_t fw[4], fx[4];
-#pragma unroll
-      for (int n = 0; n < 4; ++n) fw[n] = __builtin_bit_cast(bf16x8_t, s_w[buf][lds_slot(wrow0[n] + r, 4 * kk + lg)]);
+      bf16x8_t fx[4];
 #pragma unroll
       for (int m = 0; m < 4; ++m) fx[m] = __builtin_bit_cast(bf16x8_t, s_x[buf][lds_slot(wm * 64 + m * 16 + r, 4 * kk + lg)]);
 #pragma unroll
-      for (int n = 0; n < 4; ++n)
+      for (int n = 0; n < NW; ++n) {
+        const bf16x8_t fw = __builtin_bit_cast(bf16x8_t, s_w[buf][lds_slot(wrow0[n] + r, 4 * kk + lg)]);
 #pragma unroll
-        for (int m = 0; m < 4; ++m) acc[n][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[n], fx[m], acc[n][m], 0, 0, 0);
+        for (int m = 0; m < 4; ++m) acc[n][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw, fx[m], acc[n][m], 0, 0, 0);
+      }
     }
-#endif
     if (more) put(buf ^ 1);
     __syncthreads();
     buf ^= 1;
@@ -453,13 +452,13 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
     const int pair = a.sorted[i];
     TO* o = (TO*)a.out + (size_t)pair * a.R;
 #pragma unroll
-    for (int n = 0; n < (GATED ? 2 : 4); ++n) {
-      const int c = c0 + (GATED ? wn * 32 + n * 16 : wn * 64 + n * 16) + 4 * lg;
+    for (int n = 0; n < (GATED ? NW / 2 : NW); ++n) {
+      const int c = c0 + wn * PER_WAVE + n * 16 + 4 * lg;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (c + j >= a.R) break;
         float v = acc[n][m][j];
-        if (GATED) v = gated_value(v, acc[n + 2][m][j], a.alpha, a.limit, a.shift);
+        if (GATED) v = gated_value(v, acc[n + NW / 2][m][j], a.alpha, a.limit, a.shift);
         stf<TO>(o + c + j, v);
       }
     }

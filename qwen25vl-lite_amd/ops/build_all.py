@@ -41,6 +41,7 @@ LIBRARIES = [
     ("attention_window", {"HD": 48, "VD": 16}),
     ("attention_window", {"HD": 16, "VD": 16}),
     ("attention_window", {"HD": 64, "VD": 32}),
+    ("attention_window", {"HD": 8, "VD": 8}),
     # the kind whose waves carry three column tiles (long prompts)
     ("attention_mfma", {"HD": 128, "BLK_CT": 3}),
     ("attention_mfma", {"HD": 48, "BLK_CT": 3}),
