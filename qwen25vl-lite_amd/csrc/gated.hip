@@ -447,7 +447,7 @@ extern "C" int qvl_qk_norm_rope_write(const void* x, long long x_stride, const v
 // ---------------------------------------------------------------------------------------
 #define SN_VPT 16
 
-template <typename TY, typename TO>
+template <typename TY, typename TO, int VPT>
 __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict__ y, int nslabs, long long slab_stride,
                                      const float* __restrict__ gain, float eps_y, float factor,
                                      const float* __restrict__ vec, const float* __restrict__ w, float eps,
@@ -458,10 +458,10 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
   // Everything a thread needs of the row is asked for before the first sum is waited for, and no load
   // stands inside a branch (the compiler would wait for each before the next): a column past the row's
   // end reads column 0 and counts as zero.
-  float val[SN_VPT], hv[SN_VPT], gv[SN_VPT], wv[SN_VPT];
+  float val[VPT], hv[VPT], gv[VPT], wv[VPT];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < SN_VPT; ++i) {
+  for (int i = 0; i < VPT; ++i) {
     const int c = threadIdx.x + i * blockDim.x;
     const bool ok = c < H;
     const int cc = ok ? c : 0;
@@ -479,7 +479,7 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
   if (y && gain) rs = factor / sqrtf(block_sum(ss, red) / (float)H + eps_y);
   float ss2 = 0.f;
 #pragma unroll
-  for (int i = 0; i < SN_VPT; ++i) {
+  for (int i = 0; i < VPT; ++i) {
     const int c = threadIdx.x + i * blockDim.x;
     float v = hv[i];
     if (y) v += gain ? (val[i] * rs) * gv[i] : val[i];
@@ -491,7 +491,7 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
   const float rs2 = 1.0f / sqrtf(block_sum(ss2, red) / (float)H + eps);
   TO* o = out + (size_t)m * H;
 #pragma unroll
-  for (int i = 0; i < SN_VPT; ++i) {
+  for (int i = 0; i < VPT; ++i) {
     const int c = threadIdx.x + i * blockDim.x;
     if (c < H) stf<TO>(o + c, (val[i] * rs2) * wv[i]);
   }
@@ -503,16 +503,22 @@ extern "C" int qvl_sandwich_norm(void* h, const void* y, int y_dtype, int nslabs
   if (M <= 0) return QVL_OK;
   if (H <= 0 || nslabs < 1 || (nslabs > 1 && y_dtype != 0) || (out && !w)) return QVL_ERR_SHAPE;
   if (H > 1024 * SN_VPT) return QVL_ERR_LIMIT;
-  int threads = (H + SN_VPT - 1) / SN_VPT;
-  threads = threads <= 256 ? 256 : (threads + 63) / 64 * 64;
+  // rows up to 4,096 wide: four values a thread (few rows are a chain of waits, and short chains end sooner)
+  const int vpt = H <= 4096 ? 4 : SN_VPT;
+  int threads = ((H + vpt - 1) / vpt + 63) / 64 * 64;
 #define LAUNCH(TY, TO)                                                                                              \
-  hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO>), dim3(M), dim3(threads), 0, stream, (float*)h, (const TY*)y,    \
-                     nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec, (const float*)w,    \
-                     eps, (TO*)out, (const int*)rows, H)
-  if (y_dtype == 0 && out_dtype == 0) LAUNCH(float, float);
-  else if (y_dtype == 0 && out_dtype == 1) LAUNCH(float, bf16_t);
-  else if (y_dtype == 1 && out_dtype == 1) LAUNCH(bf16_t, bf16_t);
-  else if (y_dtype == 1 && out_dtype == 0) LAUNCH(bf16_t, float);
+  if (vpt == 4)                                                                                                     \
+    hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO, 4>), dim3(M), dim3(threads), 0, stream, (float*)h,             \
+                       (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec,     \
+                       (const float*)w, eps, (TO*)out, (const int*)rows, H);                                        \
+  else                                                                                                              \
+    hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO, SN_VPT>), dim3(M), dim3(threads), 0, stream, (float*)h,        \
+                       (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec,     \
+                       (const float*)w, eps, (TO*)out, (const int*)rows, H)
+  if (y_dtype == 0 && out_dtype == 0) { LAUNCH(float, float); }
+  else if (y_dtype == 0 && out_dtype == 1) { LAUNCH(float, bf16_t); }
+  else if (y_dtype == 1 && out_dtype == 1) { LAUNCH(bf16_t, bf16_t); }
+  else if (y_dtype == 1 && out_dtype == 0) { LAUNCH(bf16_t, float); }
   else return QVL_ERR_DTYPE;
 #undef LAUNCH
   return qvl_launch_status();

@@ -465,6 +465,153 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
   }
 }
 
+// The same product with the fetches going straight from memory into LDS (global_load_lds_dwordx4: lane l
+// of a wave puts its 16 bytes at M0 + 16 l), up to ST_STAGES - 1 steps of K ahead of the step that is
+// multiplied, through ST_STAGES stages of LDS.  No register holds data on its way, so the waves can carry 128 x 256 tiles (8 tiles
+// of 16 rows of W each: 32 products from 12 operand reads a step) and a fetch is hidden by the steps before
+// it rather than by other waves.  Chunk c of row rho lies at place c ^ ((rho >> 2) & 3) of the row (the 16
+// lanes of an operand read hit all banks), so the lane that fills place s of row rho fetches chunk
+// s ^ ((rho >> 2) & 3).  Nothing can be replaced by zeros on this way: rows that do not exist are read from
+// rows that do (their sums are not stored), and K must be a multiple of 32.  Offsets within x and within an
+// expert's W are 32-bit.
+#define ST_K 32
+#define ST_NW 8
+#define ST_M 128
+#define ST_N (32 * ST_NW)
+#ifndef ST_STAGES
+#define ST_STAGES 5                                    // steps of K in LDS: one being multiplied, the others on their way
+#endif
+#define ST_X_SLOTS (ST_M * 4)                          // 16-byte places of x in a stage
+#define ST_SLOTS ((ST_M + ST_N) * 4)                   // and of x and W together
+#define ST_WAVE_LOADS (ST_SLOTS / 64 / 4)              // loads of 1 KB a wave issues a step
+
+__device__ __forceinline__ void fetch16_to_lds(const void* base, uint32_t lane_bytes, uint32_t lds_at) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_bytes), "s"(base), "s"(lds_at)
+               : "memory", "m0");
+}
+// Wait until at most N of this wave's fetches are outstanding (they finish in order).
+template <int N>
+__device__ __forceinline__ void wait_fetches() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
+template <bool GATED, typename TO>
+__global__ __launch_bounds__(256) void moe_stream_kernel(ExpertArgs a, int tiles_m, int tiles_n) {
+  __shared__ __attribute__((aligned(16))) uint4 stage[ST_STAGES][ST_SLOTS];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, lg = lane >> 4, r = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int super = (idx >> 5) * 8 + xcd, inner = idx & 31;
+  const int supers_m = (tiles_m + 3) / 4;
+  const int tile_n = (super / supers_m) * 8 + (inner >> 2);
+  int tile = (super % supers_m) * 4 + (inner & 3);
+  if (tile >= tiles_m || tile_n >= tiles_n) return;
+  int e = 0, first = 0, last = 0;
+  for (; e < a.E; ++e) {
+    first = a.offsets[e];
+    last = a.offsets[e + 1];
+    const int nt = (last - first + ST_M - 1) / ST_M;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (e >= a.E) return;
+  first += tile * ST_M;
+  constexpr int HALF = ST_N / 2;
+  constexpr int OUT_COLS = GATED ? HALF : ST_N;
+  const int c0 = tile_n * OUT_COLS;
+  const int rows_w = GATED ? 2 * a.R : a.R;
+  const bf16_t* we = (const bf16_t*)a.w + (size_t)e * rows_w * a.K;
+
+  // this wave's fetches of a step: places wave * ST_WAVE_LOADS * 64 ... of the stage, 64 a fetch
+  uint32_t from[ST_WAVE_LOADS];      // byte offset of this lane's 16 bytes at K = 0, within x or within W_e
+#pragma unroll
+  for (int j = 0; j < ST_WAVE_LOADS; ++j) {
+    const int place = (wave * ST_WAVE_LOADS + j) * 64 + lane;
+    if (place < ST_X_SLOTS) {
+      const int row = place >> 2, ch = (place & 3) ^ ((row >> 2) & 3);
+      const int i = first + row;
+      const int pair = a.sorted[i < last ? i : first];
+      from[j] = (uint32_t)(((size_t)(pair / a.div) * a.ldx + 8 * ch) * 2);
+    } else {
+      const int row = (place - ST_X_SLOTS) >> 2, ch = (place & 3) ^ ((row >> 2) & 3);
+      int wrow;
+      if (GATED) wrow = row < HALF ? c0 + row : a.R + c0 + (row - HALF);
+      else wrow = c0 + row;
+      const bool ok = GATED ? (c0 + (row % HALF) < a.R) : (wrow < a.R);
+      from[j] = (uint32_t)(((size_t)(ok ? wrow : 0) * a.K + 8 * ch) * 2);
+    }
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)&stage[0][0];
+  auto issue = [&](int step) {
+    const uint32_t at = lds0 + (uint32_t)(step % ST_STAGES) * (ST_SLOTS * 16) + (uint32_t)wave * (ST_WAVE_LOADS * 1024);
+    const uint32_t k_bytes = (uint32_t)step * (ST_K * 2);
+#pragma unroll
+    for (int j = 0; j < ST_WAVE_LOADS; ++j) {
+      // a fetch lies wholly in x's places or wholly in W's: the same base for all its lanes
+      const bool is_x = (wave * ST_WAVE_LOADS + j) * 64 < ST_X_SLOTS;
+      fetch16_to_lds(is_x ? (const void*)a.x : (const void*)we, from[j] + k_bytes, at + j * 1024);
+    }
+  };
+  f32x4_t acc[ST_NW][4];
+#pragma unroll
+  for (int n = 0; n < ST_NW; ++n)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[n][m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  constexpr int PER_WAVE = GATED ? 8 * ST_NW : 16 * ST_NW;
+  int wrow0[ST_NW];
+#pragma unroll
+  for (int n = 0; n < ST_NW; ++n)
+    wrow0[n] = GATED ? (n < ST_NW / 2 ? wn * PER_WAVE + n * 16 : HALF + wn * PER_WAVE + (n - ST_NW / 2) * 16) : wn * PER_WAVE + n * 16;
+
+  const int steps = a.K / ST_K;
+#pragma unroll
+  for (int i = 0; i < ST_STAGES - 1; ++i)
+    if (i < steps) issue(i);
+  for (int s = 0; s < steps; ++s) {
+    // the steps after s that have been asked for may still be on their way: ST_STAGES - 2 of them, fewer at the end
+    const int ahead = steps - 1 - s < ST_STAGES - 2 ? steps - 1 - s : ST_STAGES - 2;
+    if (ahead >= 3) wait_fetches<3 * ST_WAVE_LOADS>();
+    else if (ahead == 2) wait_fetches<2 * ST_WAVE_LOADS>();
+    else if (ahead == 1) wait_fetches<ST_WAVE_LOADS>();
+    else wait_fetches<0>();
+    __syncthreads();                                    // every wave's part of step s is there, and step s - 1 has been multiplied
+    if (s + ST_STAGES - 1 < steps) issue(s + ST_STAGES - 1);
+    const uint4* sx = stage[s % ST_STAGES];
+    const uint4* sw = sx + ST_X_SLOTS;
+    bf16x8_t fx[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int row = wm * 64 + m * 16 + r;
+      fx[m] = __builtin_bit_cast(bf16x8_t, sx[row * 4 + (lg ^ ((row >> 2) & 3))]);
+    }
+#pragma unroll
+    for (int n = 0; n < ST_NW; ++n) {
+      const int row = wrow0[n] + r;
+      const bf16x8_t fw = __builtin_bit_cast(bf16x8_t, sw[row * 4 + (lg ^ ((row >> 2) & 3))]);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) acc[n][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw, fx[m], acc[n][m], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const int i = first + wm * 64 + m * 16 + r;
+    if (i >= last) continue;
+    const int pair = a.sorted[i];
+    TO* o = (TO*)a.out + (size_t)pair * a.R;
+#pragma unroll
+    for (int n = 0; n < (GATED ? ST_NW / 2 : ST_NW); ++n) {
+      const int c = c0 + wn * PER_WAVE + n * 16 + 4 * lg;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (c + j >= a.R) break;
+        float v = acc[n][m][j];
+        if (GATED) v = gated_value(v, acc[n + ST_NW / 2][m][j], a.alpha, a.limit, a.shift);
+        stf<TO>(o + c + j, v);
+      }
+    }
+  }
+}
+
 // x_dtype / out_dtype: 0 float32, 1 bfloat16.  float32 operands write float32; bfloat16 operands
 // write either.  The matrix-core kernel runs for bfloat16 with K a multiple of 8 and rows of x on
 // 16-byte boundaries; `big_tiles` asks for the kernel with tiles of 128 pairs through LDS (many pairs an expert).
@@ -478,6 +625,24 @@ extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const 
   a.P = P; a.E = E; a.R = R; a.K = K; a.div = div; a.gated = gated; a.alpha = alpha; a.limit = limit; a.shift = shift;
   if (x_dtype == 1 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0) {
     if (out_dtype != 0 && out_dtype != 1) return QVL_ERR_DTYPE;
+#ifndef MOE_NO_STREAM
+    const unsigned long long x_rows = (unsigned long long)((P + div - 1) / div);
+    if (big_tiles && K % ST_K == 0 && x_rows * (unsigned long long)ldx * 2 < 0xffffff00ull &&
+        (unsigned long long)(gated ? 2 * R : R) * K * 2 < 0xffffff00ull) {
+      const int cols = gated ? ST_N / 2 : ST_N;
+      const int tiles_m = P / ST_M + (E < P ? E : P), tiles_n = (R + cols - 1) / cols;
+      if ((long long)tiles_m * tiles_n > 0x7ffffff0ll) return QVL_ERR_LIMIT;
+      const int supers = ((tiles_m + 3) / 4) * ((tiles_n + 7) / 8);
+      const dim3 tgrid((unsigned)((supers + 7) / 8) * 8 * 32);
+      if (gated && out_dtype == 1)
+        hipLaunchKernelGGL((moe_stream_kernel<true, bf16_t>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      else if (gated) hipLaunchKernelGGL((moe_stream_kernel<true, float>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      else if (out_dtype == 1)
+        hipLaunchKernelGGL((moe_stream_kernel<false, bf16_t>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      else hipLaunchKernelGGL((moe_stream_kernel<false, float>), tgrid, dim3(256), 0, stream, a, tiles_m, tiles_n);
+      return qvl_launch_status();
+    }
+#endif
     if (big_tiles) {
       const int cols = gated ? TILE_N / 2 : TILE_N;
       const int tiles_m = P / TILE_M + (E < P ? E : P), tiles_n = (R + cols - 1) / cols;
@@ -515,24 +680,53 @@ extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const 
 // out[n, :] = sum over k of wts[n, k] * y[n top + k, :], in the order of k, plus `extra[n, :]` (what
 // a shared expert gave: float32 or bfloat16, or float32 slabs added in order; null: nothing).
 // ---------------------------------------------------------------------------------------
-template <typename TY, typename TX>
+// four consecutive values as float32
+template <typename T> __device__ __forceinline__ float4 ld4(const T* p);
+template <> __device__ __forceinline__ float4 ld4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 ld4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                __uint_as_float(v.y & 0xffff0000u)};
+}
+
+// VEC 4: a thread owns four neighbouring columns of one token (H a multiple of 4); VEC 1: one column.
+// Its loads are all on their way before the first is used.
+template <typename TY, typename TX, int VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const TY* __restrict__ y, const float* __restrict__ wts,
                                                           const TX* __restrict__ extra, int nslabs, long long slab_stride,
                                                           float* __restrict__ out, int top, int H) {
-  // a thread owns one column of one token: its loads are all on their way before the first is used
   const size_t n = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * VEC;
   if (c >= H) return;
   const float* wr = wts + n * top;
-  float v = 0.f;
+  if (VEC == 4) {
+    float4 v = float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
-  for (int k = 0; k < top; ++k) v += wr[k] * ldf<TY>(y + (n * top + k) * (size_t)H + c);
-  if (extra) {
-    float x = ldf<TX>(extra + n * H + c);
-    for (int s = 1; s < nslabs; ++s) x += ldf<TX>(extra + (size_t)s * slab_stride + n * H + c);
-    v += x;
+    for (int k = 0; k < top; ++k) {
+      const float4 t = ld4<TY>(y + (n * top + k) * (size_t)H + c);
+      const float w = wr[k];
+      v.x += w * t.x; v.y += w * t.y; v.z += w * t.z; v.w += w * t.w;
+    }
+    if (extra) {
+      float4 x = ld4<TX>(extra + n * H + c);
+      for (int s = 1; s < nslabs; ++s) {
+        const float4 t = ld4<TX>(extra + (size_t)s * slab_stride + n * H + c);
+        x.x += t.x; x.y += t.y; x.z += t.z; x.w += t.w;
+      }
+      v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+    }
+    *reinterpret_cast<float4*>(out + n * H + c) = v;
+  } else {
+    float v = 0.f;
+#pragma unroll 8
+    for (int k = 0; k < top; ++k) v += wr[k] * ldf<TY>(y + (n * top + k) * (size_t)H + c);
+    if (extra) {
+      float x = ldf<TX>(extra + n * H + c);
+      for (int s = 1; s < nslabs; ++s) x += ldf<TX>(extra + (size_t)s * slab_stride + n * H + c);
+      v += x;
+    }
+    out[n * H + c] = v;
   }
-  out[n * H + c] = v;
 }
 
 extern "C" int qvl_moe_combine(const void* y, int y_dtype, const void* wts, const void* extra, int extra_dtype,
@@ -540,13 +734,18 @@ extern "C" int qvl_moe_combine(const void* y, int y_dtype, const void* wts, cons
   if (N <= 0) return QVL_OK;
   if (top <= 0 || H <= 0 || nslabs < 1 || (nslabs > 1 && extra_dtype != 0)) return QVL_ERR_SHAPE;
 #define LAUNCH(TY, TX)                                                                                         \
-  hipLaunchKernelGGL((moe_combine_kernel<TY, TX>), dim3(N, (H + 255) / 256), dim3(256), 0, stream, (const TY*)y,   \
-                     (const float*)wts,                                                                            \
-                     (const TX*)extra, nslabs, slab_stride, (float*)out, top, H)
-  if (y_dtype == 0 && extra_dtype == 0) LAUNCH(float, float);
-  else if (y_dtype == 0 && extra_dtype == 1) LAUNCH(float, bf16_t);
-  else if (y_dtype == 1 && extra_dtype == 0) LAUNCH(bf16_t, float);
-  else if (y_dtype == 1 && extra_dtype == 1) LAUNCH(bf16_t, bf16_t);
+  if (vec4)                                                                                                        \
+    hipLaunchKernelGGL((moe_combine_kernel<TY, TX, 4>), dim3(N, (H / 4 + 255) / 256), dim3(256), 0, stream,          \
+                       (const TY*)y, (const float*)wts, (const TX*)extra, nslabs, slab_stride, (float*)out, top, H); \
+  else                                                                                                             \
+    hipLaunchKernelGGL((moe_combine_kernel<TY, TX, 1>), dim3(N, (H + 255) / 256), dim3(256), 0, stream,              \
+                       (const TY*)y, (const float*)wts, (const TX*)extra, nslabs, slab_stride, (float*)out, top, H)
+  const bool vec4 = H % 4 == 0 && slab_stride % 4 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)extra % 16) == 0 &&
+                    ((uintptr_t)out % 16) == 0;
+  if (y_dtype == 0 && extra_dtype == 0) { LAUNCH(float, float); }
+  else if (y_dtype == 0 && extra_dtype == 1) { LAUNCH(float, bf16_t); }
+  else if (y_dtype == 1 && extra_dtype == 0) { LAUNCH(bf16_t, float); }
+  else if (y_dtype == 1 && extra_dtype == 1) { LAUNCH(bf16_t, bf16_t); }
   else return QVL_ERR_DTYPE;
 #undef LAUNCH
   return qvl_launch_status();

@@ -144,11 +144,13 @@ def test_router(e, top, groups, keep):
 
 
 @pytest.mark.parametrize("dtype, width, ff", [(torch.float32, 56, 24), (torch.bfloat16, 64, 40), (torch.bfloat16, 56, 24),
-                                              (torch.bfloat16, 50, 11), (torch.float32, 50, 11)])
+                                              (torch.bfloat16, 50, 11), (torch.float32, 50, 11), (torch.bfloat16, 128, 96),
+                                              (torch.bfloat16, 96, 160)])
 @pytest.mark.parametrize("rows", [3, 150, 700])
 def test_routed_experts_alone(dtype, width, ff, rows, tmp_path):
     """Few rows (a tile of 16 pairs an expert) and many (one and several tiles of 128), widths on and off the matrix
-    cores' steps, in float32 and bfloat16, with a shared expert and clamps that bite."""
+    cores' steps and the steps of 32 that the kernel with fetches straight into LDS takes (a few and many of
+    them), in float32 and bfloat16, with a shared expert and clamps that bite."""
     mlp = du.moe(6, 3, ff, 0.8, groups=(3, 2), scale=1.3, shared=(ff + 8, 0.5))
     lay = du.layer(du.attention(1, 1, 16, 16, 16, scale=0.25), mlp)
     runner, block, t = _one_layer(tmp_path, lay, dtype=dtype, width=width)
