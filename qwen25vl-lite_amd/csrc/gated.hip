@@ -497,6 +497,45 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
   }
 }
 
+// The same for rows of up to 4,096 values whose width is a multiple of 4: a thread owns four neighbouring
+// columns and asks for them 16 bytes at a time (8 of a bfloat16 addend).
+template <typename TY, typename TO>
+__global__ void sandwich_norm_vec4_kernel(float* __restrict__ h, const TY* __restrict__ y, int nslabs, long long slab_stride,
+                                          const float* __restrict__ gain, float eps_y, float factor,
+                                          const float* __restrict__ vec, const float* __restrict__ w, float eps,
+                                          TO* __restrict__ out, const int* __restrict__ rows, int H) {
+  __shared__ float red[17];
+  const int m = blockIdx.x, n = rows ? rows[m] : m;
+  const int c = 4 * threadIdx.x;
+  const bool ok = c < H;
+  const int cc = ok ? c : 0;            // a thread past the row's end reads its start and counts as zero
+  float* hr = h + (size_t)n * H;
+  float4 v = float4{0.f, 0.f, 0.f, 0.f};
+  if (y) {
+    v = ldv4<TY>(y + (size_t)n * H + cc);
+    for (int s = 1; s < nslabs; ++s) {
+      const float4 t = ldv4<TY>(y + (size_t)s * slab_stride + (size_t)n * H + cc);
+      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+    }
+  }
+  float4 hv = ldv4<float>(hr + cc);
+  const float4 add = vec ? ldv4<float>(vec + cc) : float4{0.f, 0.f, 0.f, 0.f};
+  const float4 gv = gain ? ldv4<float>(gain + cc) : float4{1.f, 1.f, 1.f, 1.f};
+  const float4 wv = w ? ldv4<float>(w + cc) : float4{1.f, 1.f, 1.f, 1.f};
+  if (!ok) { v = float4{0.f, 0.f, 0.f, 0.f}; hv = v; }
+  float rs = 1.0f;
+  if (y && gain) rs = factor / sqrtf(block_sum(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w, red) / (float)H + eps_y);
+  float4 t;
+  if (y && gain) t = float4{(v.x * rs) * gv.x, (v.y * rs) * gv.y, (v.z * rs) * gv.z, (v.w * rs) * gv.w};
+  else t = v;
+  t = float4{hv.x + add.x + t.x, hv.y + add.y + t.y, hv.z + add.z + t.z, hv.w + add.w + t.w};
+  if (!ok) t = float4{0.f, 0.f, 0.f, 0.f};
+  if (ok && !rows && (y || vec)) stv4<float>(hr + c, t);
+  if (!out) return;
+  const float rs2 = 1.0f / sqrtf(block_sum(t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w, red) / (float)H + eps);
+  if (ok) stv4<TO>(out + (size_t)m * H + c, float4{(t.x * rs2) * wv.x, (t.y * rs2) * wv.y, (t.z * rs2) * wv.z, (t.w * rs2) * wv.w});
+}
+
 extern "C" int qvl_sandwich_norm(void* h, const void* y, int y_dtype, int nslabs, long long slab_stride, const void* gain,
                                  float eps_y, float factor, const void* vec, const void* w, float eps, void* out,
                                  int out_dtype, const void* rows, int M, int H, hipStream_t stream) {
@@ -506,8 +545,14 @@ extern "C" int qvl_sandwich_norm(void* h, const void* y, int y_dtype, int nslabs
   // rows up to 4,096 wide: four values a thread (few rows are a chain of waits, and short chains end sooner)
   const int vpt = H <= 4096 ? 4 : SN_VPT;
   int threads = ((H + vpt - 1) / vpt + 63) / 64 * 64;
+  const bool vec4 = H % 4 == 0 && H <= 4096 && slab_stride % 4 == 0 &&
+                    (((uintptr_t)h | (uintptr_t)y | (uintptr_t)gain | (uintptr_t)vec | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
 #define LAUNCH(TY, TO)                                                                                              \
-  if (vpt == 4)                                                                                                     \
+  if (vec4)                                                                                                         \
+    hipLaunchKernelGGL((sandwich_norm_vec4_kernel<TY, TO>), dim3(M), dim3((H / 4 + 63) / 64 * 64), 0, stream,       \
+                       (float*)h, (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor,             \
+                       (const float*)vec, (const float*)w, eps, (TO*)out, (const int*)rows, H);                     \
+  else if (vpt == 4)                                                                                                \
     hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO, 4>), dim3(M), dim3(threads), 0, stream, (float*)h,             \
                        (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec,     \
                        (const float*)w, eps, (TO*)out, (const int*)rows, H);                                        \
