@@ -85,8 +85,8 @@ def dazapel_config(layers, size="7b", experts=32, top=6, window=1024, keep_first
 
     def mixer(i):
         m = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
-             "rot": {"base": 500000.0, "dims": hd // 2,
-                     "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+             "rot": {"base": 1000000.0, "dims": hd // 2,
+                     "scaling": {"factor": 8.0, "original": 8192, "fast": 16.0, "slow": 2.0}}}
         if i % 2:
             m["mask"] = {"size": window, "keep_first": keep_first}
         return m

@@ -47,11 +47,11 @@ RAMP = {"factor": 8.0, "original": 32, "fast": 4.0, "slow": 0.5}
 MIXED = config(72, 203, [
     layer(attention(4, 2, 16, 24, 8, base=500.0, scaling=RAMP, scale=0.7, mask=(9, 3)),
           moe(6, 2, 40, 1.0, groups=(3, 2), scale=1.5, shared=(56, 0.8))),
-    layer(attention(6, 3, 20, 12, 20, base=10000.0, scale=0.5, mask=(21, 0)),
+    layer(attention(6, 2, 20, 12, 20, base=10000.0, scale=0.5, mask=(21, 0)),
           moe(8, 3, 24, 2.0, groups=(4, 2), scale=0.7)),
     layer(attention(2, 2, 32, 32, 16, base=80.0, scaling={"factor": 2.0, "original": 16, "fast": 2.0, "slow": 1.0},
                     scale=0.4)),
-    layer(attention(3, 1, 48, 16, 48, base=2000.0, scale=0.3, mask=(40, 20)),
+    layer(attention(3, 1, 48, 16, 48, base=2000.0, scale=0.3, mask=(37, 18)),
           moe(4, 4, 32, 0.6, groups=(1, 1), scale=2.0, shared=(16, 1.5))),
 ], eps=1e-5, mult=0.4, loop=(1, 3, 3))
 
