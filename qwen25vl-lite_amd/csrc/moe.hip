@@ -13,9 +13,9 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 
 // ---------------------------------------------------------------------------------------
 // Router.  z [N, E] float32 logits.  s = sigmoid(z) (score_fn 0) or softmax(z) over the experts
-// (score_fn 1).  The experts form `groups` equal groups of neighbours; a group's score is the sum of
-// its two largest s (of its one, if it has one); only experts of the `keep` best groups can be
-// chosen; the `top` largest s among those are the choice (ties: the lower index).  Weights: the
+// (score_fn 1).  Experts e with the same e / (E / groups) are one group, ranked by the sum of its
+// top two s (its only one, if it has one member); the choice is the `top` highest s among the members
+// of the `keep` highest-ranked groups (ties: the lower index).  Weights: the
 // chosen s divided by (their sum + floor) if `normalize`, times `scale`.
 // One wave per token; E <= 512, groups <= 64.
 // ---------------------------------------------------------------------------------------

@@ -10,7 +10,7 @@ by adding its vector (a row of ``loop.step``) to the sum.
   frequencies stretched by a ramp over the channel index and cosines and sines scaled (``rot.scaling``:
   ``factor``, ``original``, ``fast``, ``slow``), then queries and keys divided by their root mean square
   per head, a fixed score scale, a sliding window that also keeps a request's first tokens visible
-  (``mask``: ``size``, ``keep_first``), the concatenated heads multiplied element by element by the sigmoid of a
+  (``mask``: ``size``, ``keep_first``), every channel of the heads' joined output scaled by the sigmoid of its own channel of a
   projection of the mixer's input, a biased output projection.
 * feed-forward ``moe``: routed experts with sigmoid scores, a choice limited to the best groups of
   neighbouring experts, weights normalised over the choice and scaled, plus a shared expert.  Every

@@ -19,7 +19,7 @@ __all__ = ["route", "sort_pairs", "expert_products", "combine", "SCORE_FUNCTIONS
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 SCORE_FUNCTIONS = {"sigmoid": 0, "softmax": 1}
-# from this many pairs per expert on (on average) the matrix-core kernel takes tiles of 64 pairs
+# from this many pairs per expert on (on average) the matrix-core kernels with tiles of 128 pairs through LDS run
 BIG_TILE_PAIRS = 32
 
 
@@ -27,9 +27,9 @@ def route(logits: torch.Tensor, top: int, groups: int = 1, keep: int = 1, scale:
           score: str = "sigmoid", normalize: bool = True, floor: float = 1e-20) -> Tuple[torch.Tensor, torch.Tensor]:
     """``(chosen int32 [N, top], weights float32 [N, top])`` from float32 router logits ``[N, E]``.
 
-    Scores are ``sigmoid`` or ``softmax`` of the logits.  The experts form ``groups`` equal groups of
-    neighbours; a group's score is the sum of its two largest scores; only experts of the ``keep``
-    best groups can be chosen, the ``top`` with the largest scores.  The weights are the chosen
+    Scores are ``sigmoid`` or ``softmax`` of the logits.  Experts ``e`` with the same ``e // (E / groups)`` are one
+    group, ranked by the sum of its top two scores; the ``top`` experts with the highest scores are
+    picked among the members of the ``keep`` highest-ranked groups.  The weights are the chosen
     scores, divided by their sum plus ``floor`` if ``normalize``, times ``scale``."""
     _dev(logits)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(),

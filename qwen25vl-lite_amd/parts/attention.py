@@ -41,8 +41,9 @@ class PagedAttention(Mixer):
     ``qk_norm_where`` (``"before"``, the default, or ``"after"`` the rotation) and ``qk_norm_weights``
     (False: the norm has no gains and the mixer no such tensors), ``value_dim`` (values of another
     width than keys), ``keep_first`` (with a window: the first so many keys of a request stay visible
-    to every later token, at their true positions), ``element_gate`` (the concatenated heads are
-    multiplied element by element by the sigmoid of a projection ``g`` of ``[heads value_dim, hidden]``),
+    to every later token; their rotation and their distance to a query are those of where they stand),
+    ``element_gate`` (channel ``c`` of the heads' joined output is scaled by ``sigmoid(g_c)``, ``g`` a
+    projection of ``[heads value_dim, hidden]``),
     ``out_bias`` (the output projection has a bias).  Any of these except the last takes the
     projection through float32 and one kernel that norms, rotates and writes the cache."""
 

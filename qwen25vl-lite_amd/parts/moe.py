@@ -2,9 +2,9 @@
 expert that every token uses.
 
 The router's logits ``z = x Wr^T`` are float32 sums.  Scores ``s`` are ``sigmoid(z)`` (or a softmax
-over the experts).  The experts form equal groups of neighbours; a group's score is the sum of its
-two largest scores; only experts of the best ``keep`` groups can be chosen, the ``top`` with the
-largest scores.  A token's result is ``sum_k w_k expert_k(x)`` with ``w`` the chosen scores over
+over the experts).  Experts ``e`` with the same ``e // (E / groups)`` are one group, ranked by the sum of its
+top two scores; the ``top`` experts with the highest scores are picked among the members of the
+``keep`` highest-ranked groups.  A token's result is ``sum_k w_k expert_k(x)`` with ``w`` the chosen scores over
 their sum, times ``scale``, plus ``shared(x)``.  Every expert is
 ``down(g sigmoid(alpha g) (u + shift))`` with ``g = min(gate(x), limit)``, ``u = clamp(up(x), +-limit)``.
 """
